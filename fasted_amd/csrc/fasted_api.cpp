@@ -1,0 +1,408 @@
+// fasted_api.cpp -- host driver and C ABI of libfasted.so (declarations: include/fasted.h).
+//
+// Host orchestration of one join, the counterpart of SimSearch::FindPairs
+// (source/findPairs.cuh:615-764): upload once, time squared norms and the join kernel with
+// device events, sort the stored pairs row-major, hand the pairs back (or write the
+// ".pairs" text file), report Results.  The resident dataset lives in process globals so
+// that reRun() can change epsilon without touching the data (source/main.cu:33,198-248).
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <climits>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "../../include/fasted.h"
+#include "join_kernels.h"
+#include "point_table.hpp"
+
+static_assert(sizeof(mmaShape) == 12, "mmaShape layout is part of the ABI");
+static_assert(sizeof(Results) == 56, "Results layout is part of the ABI");
+static_assert(offsetof(Results, pairsFound) == 16 && offsetof(Results, inputProblemShape) == 32 &&
+                  offsetof(Results, paddedProblemShape) == 44,
+              "Results layout is part of the ABI");
+static_assert(sizeof(FastedPair) == 8, "pair record is 8 bytes");
+
+namespace {
+
+std::string g_error;
+std::string g_outDir;
+
+struct HipFailure : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw HipFailure(std::string(what) + ": " + hipGetErrorString(e));
+}
+#define HIP_CHECK(expr) hip_check((expr), #expr)
+
+int round_up(long long v, int m) { return (int)(((v + m - 1) / m) * m); }
+
+bool quiet() {
+    static const bool q = [] {
+        const char* v = std::getenv("FASTED_QUIET");
+        return v && *v && *v != '0';
+    }();
+    return q;
+}
+
+// Small device workspace that survives between calls: counters and a squared-norm buffer.
+struct Workspace {
+    unsigned long long* counters = nullptr;
+    float* sums = nullptr;
+    size_t sumsCap = 0;
+
+    void ensure(size_t n) {
+        if (!counters) HIP_CHECK(hipMalloc(&counters, 4 * sizeof(unsigned long long)));
+        if (n > sumsCap) {
+            if (sums) HIP_CHECK(hipFree(sums));
+            sums = nullptr;
+            sumsCap = 0;
+            HIP_CHECK(hipMalloc(&sums, n * sizeof(float)));
+            sumsCap = n;
+        }
+    }
+    void release() {
+        if (counters) (void)hipFree(counters);
+        if (sums) (void)hipFree(sums);
+        counters = nullptr;
+        sums = nullptr;
+        sumsCap = 0;
+    }
+} g_ws;
+
+struct EventTimer {
+    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    EventTimer() {
+        for (auto& e : ev) HIP_CHECK(hipEventCreate(&e));
+    }
+    ~EventTimer() {
+        for (auto& e : ev)
+            if (e) (void)hipEventDestroy(e);
+    }
+    float ms(int a, int b) {
+        float t = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&t, ev[a], ev[b]));
+        return t;
+    }
+};
+
+void validate_shape(long long n, int d, long long ld) {
+    if (n < 1) throw std::invalid_argument("number of points must be at least 1");
+    if (n > (long long)INT_MAX - 2 * fasted::kTile) throw std::invalid_argument("number of points exceeds int range");
+    if (d < 1) throw std::invalid_argument("dimensionality must be at least 1");
+    const long long dPad = round_up(d, fasted::kSlabK);
+    if (ld % 8 != 0) throw std::invalid_argument("row stride must be a multiple of 8 halves (16 bytes)");
+    if (ld < dPad) throw std::invalid_argument("row stride must cover the dimensionality rounded up to 64");
+    if ((ld / 8) * fasted::kTile >= (1ll << 31)) throw std::invalid_argument("row stride too large");
+}
+
+// The timed region of the reference (source/findPairs.cuh:625-697): squared norms, then
+// queue/pair-counter reset and the join kernel; then counters come back and the stored pairs
+// are sorted outside the TFLOPS window.
+void join_on_device(const void* dPoints, long long n, int d, long long ld, double epsilon, float* dSums, void* dPairs,
+                    unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats) {
+    validate_shape(n, d, ld);
+    if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
+    const int dPad = round_up(d, fasted::kSlabK);
+    g_ws.ensure((size_t)n);
+    float* sums = dSums ? dSums : g_ws.sums;
+    if ((flags & FASTED_SKIP_SUMS) && !dSums) throw std::invalid_argument("FASTED_SKIP_SUMS needs d_sums");
+
+    EventTimer t;
+    HIP_CHECK(hipEventRecord(t.ev[0], stream));
+    if (!(flags & FASTED_SKIP_SUMS)) HIP_CHECK(fasted::launch_sum_squared(dPoints, ld, (int)n, dPad, sums, stream));
+    HIP_CHECK(hipEventRecord(t.ev[1], stream));
+
+    fasted::JoinLaunch jl;
+    jl.points = dPoints;
+    jl.ld = ld;
+    jl.n = (int)n;
+    jl.dPad = dPad;
+    jl.eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
+    jl.sums = sums;
+    jl.counters = g_ws.counters;
+    jl.pairs = dPairs;
+    jl.cap = cap;
+    jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
+    HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, stream));
+    HIP_CHECK(fasted::launch_join(jl, stream));
+    HIP_CHECK(hipEventRecord(t.ev[2], stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+
+    unsigned long long c[4] = {0, 0, 0, 0};
+    HIP_CHECK(hipMemcpy(c, g_ws.counters, sizeof c, hipMemcpyDeviceToHost));
+    float sortMs = 0.f;
+    if ((flags & FASTED_SORT_PAIRS) && c[1] > 1) {
+        const auto w0 = std::chrono::steady_clock::now();
+        HIP_CHECK(fasted::sort_pairs_row_major(dPairs, c[1], stream));
+        sortMs = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
+    }
+    if (stats) {
+        stats->sumSquaredMs = t.ms(0, 1);
+        stats->joinMs = t.ms(1, 2);
+        stats->sortMs = sortMs;
+        stats->paddedN = round_up(n, fasted::kTile);
+        stats->paddedD = dPad;
+        stats->tiles = c[3];
+        stats->pairsFound = c[0];
+        stats->pairsStored = c[1];
+    }
+}
+
+// ---- resident dataset of the reference-compatible entry points -------------------------
+struct Resident {
+    fasted::PointTable table;
+    void* dPoints = nullptr;
+    bool uploaded = false;
+    void drop_device() {
+        if (dPoints) (void)hipFree(dPoints);
+        dPoints = nullptr;
+        uploaded = false;
+    }
+} g_res;
+
+std::string output_dir() {
+    if (!g_outDir.empty()) return g_outDir;
+    const char* env = std::getenv("FASTED_PAIRS_DIR");
+    return env && *env ? std::string(env) : std::string(".");
+}
+
+void write_pairs_text(const std::string& path, const std::vector<FastedPair>& pairs) {
+    std::FILE* f = std::fopen(path.c_str(), "w");
+    if (!f) throw std::ios_base::failure("Failed to open output file: " + path);
+    // "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54
+    for (const FastedPair& p : pairs) std::fprintf(f, "%d, %d\n", p.QueryPoint, p.CandidatePoint);
+    std::fclose(f);
+}
+
+Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, const std::string& datasetName) {
+    const auto wall0 = std::chrono::steady_clock::now();
+    const fasted::PointTable& tb = g_res.table;
+    if (tb.empty()) throw std::runtime_error("no dataset is resident: call runFromFile or runFromExponentialDataset first");
+    HIP_CHECK(hipSetDevice(0));
+    const size_t bytes = tb.bits.size() * sizeof(uint16_t);
+    if (!skipUpload || !g_res.uploaded) {
+        g_res.drop_device();
+        if (!quiet()) std::printf("Allocating %zu bytes for the points (queries and candidates share one copy)\n", bytes);
+        HIP_CHECK(hipMalloc(&g_res.dPoints, bytes));
+        HIP_CHECK(hipMemcpy(g_res.dPoints, tb.bits.data(), bytes, hipMemcpyHostToDevice));
+        g_res.uploaded = true;
+    }
+    HIP_CHECK(hipDeviceSynchronize());
+
+    // Pair buffer: N*256 records, shrunk to what the device can still hold
+    // (source/findPairs.cuh:644-647, source/pair.cuh:69-85).  Half of the free memory is the
+    // limit here because the row-major sort needs a second buffer of the stored size.
+    unsigned long long maxPairs = (unsigned long long)tb.n * 256ull;
+    size_t freeB = 0, totalB = 0;
+    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
+    const unsigned long long fit = (unsigned long long)(freeB / 2) / sizeof(FastedPair);
+    if (maxPairs > fit) {
+        std::printf("Failed to allocate enough space for %llu pairs. Reducing max number of pairs to %llu\n", maxPairs,
+                    fit);
+        maxPairs = fit;
+    }
+    void* dPairs = nullptr;
+    HIP_CHECK(hipMalloc(&dPairs, (size_t)(maxPairs ? maxPairs : 1) * sizeof(FastedPair)));
+
+    FastedJoinStats st{};
+    std::vector<FastedPair> pairs;
+    try {
+        join_on_device(g_res.dPoints, tb.n, tb.dPad, tb.dPad, epsilon, nullptr, dPairs, maxPairs, FASTED_SORT_PAIRS,
+                       nullptr, &st);
+        if (!quiet()) {
+            std::printf("Number of pairs found %llu\n", st.pairsFound);
+            std::printf("Number of pairs stored %llu\n", st.pairsStored);
+        }
+        // the pairs always leave the device, saved or not (source/findPairs.cuh:705-714)
+        pairs.resize((size_t)st.pairsStored);
+        if (st.pairsStored)
+            HIP_CHECK(hipMemcpy(pairs.data(), dPairs, pairs.size() * sizeof(FastedPair), hipMemcpyDeviceToHost));
+    } catch (...) {
+        (void)hipFree(dPairs);
+        throw;
+    }
+    HIP_CHECK(hipFree(dPairs));
+    if (savePairs) {
+        const std::string path = output_dir() + "/" + datasetName + "_" + std::to_string(epsilon) + ".pairs";
+        std::cout << "Output file is: " << path << std::endl;
+        write_pairs_text(path, pairs);
+    }
+    const double totalTime = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
+    const float kernelSec = (st.sumSquaredMs + st.joinMs) / 1000.0f;
+    // unpadded shape: padded zeros are not useful work (source/findPairs.cuh:745-747)
+    const float tflops = static_cast<float>(tb.n) * tb.n * tb.d * 2 / kernelSec / 1e12f;
+    if (!quiet()) {
+        std::printf("Total Elapsed time: %f seconds\n", totalTime);
+        std::printf("Total Kernel Elapsed time: %f seconds\n", kernelSec);
+        std::printf("SumSquared Kernel Elapsed time: %f seconds\n", st.sumSquaredMs / 1000.0f);
+        std::printf("FindPairs Kernel Elapsed time: %f seconds\n", st.joinMs / 1000.0f);
+        std::printf("Pairs sort Elapsed time: %f seconds\n", st.sortMs / 1000.0f);
+        std::printf("Pairs found: %llu\n", st.pairsFound);
+        std::printf("Estimated TFLOPS %.3f\n", tflops);
+        std::fflush(stdout);
+    }
+    Results r;
+    r.totalTime = static_cast<float>(totalTime);
+    r.TFLOPS = tflops;
+    r.pairsFound = st.pairsFound;
+    r.pairsStored = st.pairsStored;
+    r.inputProblemShape = mmaShape{tb.n, tb.n, tb.d};
+    r.paddedProblemShape = mmaShape{tb.nPad, tb.nPad, tb.dPad};
+    return r;
+}
+
+// Shared body of the three run entry points, the counterpart of run() in
+// source/main.cu:198-248: failures are printed and end the process, as there.
+Results run_source(fasted::PointSource* src, double epsilon, bool savePairs) {
+    try {
+        std::string name;
+        if (src) {
+            name = src->name();
+            if (!quiet()) std::cout << "Building point list" << std::endl;
+            g_res.table = fasted::build_point_table(*src, fasted::kSlabK, fasted::kTile);
+            g_res.uploaded = false;
+            if (!quiet()) {
+                std::cout << "Number of points is: " << g_res.table.n << std::endl;
+                std::cout << "Padding with " << g_res.table.nPad - g_res.table.n << " points" << std::endl;
+            }
+        }
+        const fasted::PointTable& tb = g_res.table;
+        if (!quiet() && !tb.empty()) {
+            std::cout << "Padded Search Dimensions:\nM: " << tb.nPad << "\nN: " << tb.nPad << "\nK: " << tb.dPad
+                      << std::endl;
+            std::cout << "Input Search Dimensions:\nM: " << tb.n << "\nN: " << tb.n << "\nK: " << tb.d << std::endl;
+        }
+        return find_pairs_resident(epsilon, savePairs, src == nullptr, name);
+    } catch (const std::exception& e) {
+        std::cout << "Error: Failed to run. " << e.what() << std::endl;
+        std::exit(EXIT_FAILURE);
+    }
+}
+
+template <typename F>
+int guarded(F&& body) {
+    try {
+        body();
+        g_error.clear();
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        (void)hipGetLastError();
+        return 1;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+Results runFromExponentialDataset(int size, int dimensionality, double lambda, double max, double epsilon,
+                                  bool savePairs) {
+    if (!quiet()) std::cout << "Running from a generated exponential dataset" << std::endl;
+    fasted::ExponentialSource src(size, dimensionality, lambda, max);
+    return run_source(&src, epsilon, savePairs);
+}
+
+Results runFromFile(const char* filename, double epsilon, bool savePairs) {
+    try {
+        const std::string path(filename ? filename : "");
+        if (!quiet()) std::cout << "Running from file: " << path << std::endl;
+        fasted::CsvSource src(path, ',');
+        return run_source(&src, epsilon, savePairs);
+    } catch (const std::exception& e) {  // the reference lets a missing file terminate the process
+        std::cout << "Error: Failed to run. " << e.what() << std::endl;
+        std::exit(EXIT_FAILURE);
+    }
+}
+
+Results reRun(double epsilon, bool savePairs) { return run_source(nullptr, epsilon, savePairs); }
+
+void releaseResources(void) {
+    g_res.drop_device();
+    g_res.table = fasted::PointTable();
+    g_ws.release();
+}
+
+int fasted_self_join_device(const void* d_points, long long n, int d, long long ld, double epsilon, float* d_sums,
+                            FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
+                            FastedJoinStats* stats) {
+    return guarded([&] {
+        if (!d_points) throw std::invalid_argument("points pointer is null");
+        join_on_device(d_points, n, d, ld, epsilon, d_sums, d_pairs, cap, flags, static_cast<hipStream_t>(stream),
+                       stats);
+    });
+}
+
+int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream) {
+    return guarded([&] {
+        if (!d_points || !d_sums) throw std::invalid_argument("null pointer");
+        validate_shape(n, d, ld);
+        HIP_CHECK(fasted::launch_sum_squared(d_points, ld, (int)n, round_up(d, fasted::kSlabK), d_sums,
+                                             static_cast<hipStream_t>(stream)));
+        HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    });
+}
+
+int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon, FastedPair* out,
+                     unsigned long long cap, unsigned long long* found, unsigned long long* stored) {
+    return guarded([&] {
+        if (!points) throw std::invalid_argument("points pointer is null");
+        if (cap > 0 && !out) throw std::invalid_argument("output buffer is null");
+        if (n < 1 || d < 1) throw std::invalid_argument("empty dataset");
+        const int dPad = round_up(d, fasted::kSlabK);
+        validate_shape(n, d, dPad);
+        void* dPoints = nullptr;
+        void* dPairs = nullptr;
+        try {
+            const size_t pitch = (size_t)dPad * 2;
+            HIP_CHECK(hipMalloc(&dPoints, (size_t)n * pitch));
+            if (dPad != d) HIP_CHECK(hipMemset(dPoints, 0, (size_t)n * pitch));
+            HIP_CHECK(hipMemcpy2D(dPoints, pitch, points, (size_t)d * 2, (size_t)d * 2, (size_t)n,
+                                  hipMemcpyHostToDevice));
+            HIP_CHECK(hipMalloc(&dPairs, (size_t)(cap ? cap : 1) * sizeof(FastedPair)));
+            FastedJoinStats st{};
+            join_on_device(dPoints, n, d, dPad, epsilon, nullptr, dPairs, cap, FASTED_SORT_PAIRS, nullptr, &st);
+            if (st.pairsStored)
+                HIP_CHECK(hipMemcpy(out, dPairs, (size_t)st.pairsStored * sizeof(FastedPair), hipMemcpyDeviceToHost));
+            if (found) *found = st.pairsFound;
+            if (stored) *stored = st.pairsStored;
+        } catch (...) {
+            if (dPoints) (void)hipFree(dPoints);
+            if (dPairs) (void)hipFree(dPairs);
+            throw;
+        }
+        (void)hipFree(dPoints);
+        (void)hipFree(dPairs);
+    });
+}
+
+int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
+    if (n < 1 || !row || !col) return 0;
+    return fasted::raster_coord(idx, n, row, col) ? 1 : 0;
+}
+
+unsigned long long fasted_raster_count(long long n) { return n < 1 ? 0ull : fasted::raster_count(n); }
+
+const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad) {
+    const fasted::PointTable& tb = g_res.table;
+    if (n) *n = tb.n;
+    if (d) *d = tb.d;
+    if (n_pad) *n_pad = tb.nPad;
+    if (d_pad) *d_pad = tb.dPad;
+    return tb.empty() ? nullptr : tb.bits.data();
+}
+
+void fasted_set_output_dir(const char* dir) { g_outDir = dir ? dir : ""; }
+
+const char* fasted_last_error(void) { return g_error.c_str(); }
+
+const char* fasted_version(void) { return "fasted-mi355x 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,37 @@
+// join_kernels.h -- host-callable launchers of the gfx950 kernels (internal to libfasted).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace fasted {
+
+constexpr int kTile = 256;       // points per tile side (queries x candidates)
+constexpr int kSlabK = 64;       // halves of K staged in LDS per pipeline stage
+constexpr int kRaster = 16;      // tiles per side of a raster square
+
+struct JoinLaunch {
+    const void* points;          // FP16 rows
+    long long ld;                // row stride in halves (multiple of 8)
+    int n;                       // real points
+    int dPad;                    // K extent, multiple of kSlabK
+    float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
+    const float* sums;           // squared norms
+    unsigned long long* counters;  // [0] found, [1] stored, [2] queue head, [3] tiles done
+    void* pairs;                 // FastedPair[cap]
+    unsigned long long cap;
+    bool epilogue;               // false: contraction only (measurement)
+};
+
+// Host mirror of the device tile order.
+unsigned long long raster_count(long long n);
+bool raster_coord(unsigned long long idx, long long n, int* row, int* col);
+
+hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream);
+hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream);
+hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
+
+// Row-major sort of `count` stored pairs (pair_sort.hip).
+hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream);
+
+}  // namespace fasted

@@ -1,0 +1,401 @@
+// join_kernels.hip -- the gfx950 (CDNA4, wave64) kernels of the epsilon self-join.
+//
+//   sum_squared_kernel   FP32 squared norm of every FP16 point; HBM-bound, 16-byte
+//                        coalesced loads, lane-group shuffle reduction.  Stands where the
+//                        reference has SumSqd::SquaredSumsKernel (source/sumSquared.cuh:53-73).
+//   join_kernel          persistent workgroups pull 256x256 tiles of the N x N distance
+//                        matrix from an atomic work queue (the reference's on-demand
+//                        rasterizer, source/rasterizer/onDemandRasterizer.cuh:78-108), form
+//                        Q.C^T with v_mfma_f32_32x32x16_f16 from XOR-swizzled, double-buffered
+//                        LDS slabs (source/findPairs.cuh:360-546 is the reference's kernel),
+//                        and run the fused test  (s_q + s_c) - 2 q.c <= eps^2
+//                        (source/warpMma.cuh:220-273) with wave-level compaction: one
+//                        atomic reservation per wave instead of one per pair
+//                        (source/pair.cuh:123-133).
+//
+// Data layout: points are row-major FP16, one point per row, row stride `ld` halves.  Both
+// MFMA operands are "row = point, 8 consecutive k per lane", so the query tile and the
+// candidate tile are staged in LDS in the same [256 rows][64 halves] form.
+#include "join_kernels.h"
+
+namespace fasted {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 512;                       // 8 waves: 2 (rows) x 4 (cols)
+constexpr int kRowBytes = kSlabK * 2;               // one LDS row of a slab: 128 B = 8 chunks of 16 B
+constexpr int kOperandBytes = kTile * kRowBytes;    // 32 KiB per operand per stage
+constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 64 KiB
+constexpr int kLdsSums = 2 * kStageBytes;           // s_q[256] then s_c[256]
+constexpr int kLdsNext = kLdsSums + 2 * kTile * 4;  // next queue index
+constexpr int kLdsBytes = kLdsNext + 16;
+constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
+constexpr int kFragRows = kWaveRows / 32, kFragCols = kWaveCols / 32;  // 4 x 2 MFMA 32x32 blocks
+
+// 16-byte chunk c of LDS row r lives at chunk slot c ^ swz(r).  Any 8 consecutive rows hit
+// 8 distinct slots, and rows r, r+8 differ in the low slot bit while sharing row parity, so
+// 16 consecutive rows at one logical chunk cover all 64 four-byte banks exactly once.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+struct Raster {
+    unsigned tilesPerDim;
+    unsigned squaresPerDim;
+    unsigned long long total;
+};
+
+__host__ __device__ inline Raster make_raster(long long n) {
+    Raster r;
+    r.tilesPerDim = (unsigned)((n + kTile - 1) / kTile);
+    r.squaresPerDim = (r.tilesPerDim + kRaster - 1) / kRaster;
+    r.total = (unsigned long long)r.squaresPerDim * r.squaresPerDim * (kRaster * kRaster);
+    return r;
+}
+
+// Queue index -> tile (row, col) in tile units.  Indices are dealt out in kRaster x kRaster
+// squares (row-major over squares, row-major inside) so that workgroups running at the same
+// time share query and candidate panels in L2 / Infinity Cache.  Tiles outside the
+// tilesPerDim grid are padding: the caller skips them.
+__host__ __device__ inline void raster_decode(const Raster& r, unsigned long long idx, unsigned* tr, unsigned* tc) {
+    const unsigned area = kRaster * kRaster;
+    unsigned long long sq = idx / area;
+    unsigned local = (unsigned)(idx % area);
+    *tr = (unsigned)(sq / r.squaresPerDim) * kRaster + local / kRaster;
+    *tc = (unsigned)(sq % r.squaresPerDim) * kRaster + local % kRaster;
+}
+
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restrict__ pts, long long ld16, int n,
+                                                          int chunksPerRow, int lanesPerRow,
+                                                          float* __restrict__ sums) {
+    const int lane = threadIdx.x & 63;
+    const long long wave = ((long long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int rowsPerWave = 64 / lanesPerRow;
+    const long long row = wave * rowsPerWave + lane / lanesPerRow;
+    const int sub = lane % lanesPerRow;
+    float acc = 0.0f;
+    if (row < n) {
+        const u32x4* p = pts + row * ld16;
+        for (int c = sub; c < chunksPerRow; c += lanesPerRow) {
+            u32x4 v = p[c];
+            half8 h = __builtin_bit_cast(half8, v);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float x = (float)h[e];
+                acc = __builtin_fmaf(x, x, acc);
+            }
+        }
+    }
+    for (int off = lanesPerRow >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (sub == 0 && row < n) sums[row] = acc;
+}
+
+__global__ void reset_counters_kernel(unsigned long long* c) {
+    if (threadIdx.x < 4) c[threadIdx.x] = 0ull;
+}
+
+// ------------------------------------------------------------------------------------------
+struct JoinParams {
+    const u32x4* pts;
+    long long ld16;  // row stride in 16-byte units
+    int n;
+    int nSlabs;
+    float eps2;
+    const float* sums;
+    unsigned long long* counters;
+    int2* pairs;
+    unsigned long long cap;
+    Raster raster;
+};
+
+// Distance test of one wave's 128x64 block.  kEdge: the tile touches the diagonal or the
+// ragged end of the dataset, so self pairs are forced and padded rows/cols are masked
+// (source/warpMma.cuh:257-259).  Returns per-lane hit bits: mask[fi] bit (fj*16 + r).
+template <bool kEdge>
+__device__ __forceinline__ void test_block(const floatx16 (&acc)[kFragRows][kFragCols], const float* sQ,
+                                           const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
+                                           int hi, int n, float eps2, unsigned (&mask)[kFragRows]) {
+#pragma unroll
+    for (int fi = 0; fi < kFragRows; ++fi) {
+        unsigned m = 0;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const floatx4 sq = *reinterpret_cast<const floatx4*>(sQ + fi * 32 + g * 8 + hi * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = g * 4 + e;
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj) {
+                    // (s_q + s_c) - 2*acc, FP32, as source/warpMma.cuh:241-242
+                    const float d2 = (sq[e] + sc[fj]) - (2.0f * acc[fi][fj][r]);
+                    bool hit = d2 <= eps2;
+                    if (kEdge) {
+                        const int q = qBase + fi * 32 + g * 8 + hi * 4 + e;
+                        hit = (hit || q == cand[fj]) && q < n && cand[fj] < n;
+                    }
+                    m |= (hit ? 1u : 0u) << (fj * 16 + r);
+                }
+            }
+        }
+        mask[fi] = m;
+    }
+}
+
+template <bool kEpilogue>
+__global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 2, wc = wave & 3;
+    const int l32 = lane & 31, hi = lane >> 5;
+
+    // copy role: 8 consecutive lanes fetch one 128-byte row segment of a slab
+    const int cpRow = tid >> 3, cpChunk = tid & 7;
+    const int cpLds = cpRow * kRowBytes + ((cpChunk ^ swz(cpRow)) << 4);  // rows +64*i keep swz
+
+    // fragment role: lane reads row l32 of a 32-row block, chunk 2*kk + hi
+    int aOff[4], bOff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        const int slot = ((kk * 2 + hi) ^ swz(l32)) << 4;
+        aOff[kk] = (wr * kWaveRows + l32) * kRowBytes + slot;
+        bOff[kk] = kOperandBytes + (wc * kWaveCols + l32) * kRowBytes + slot;
+    }
+
+    float* const sQ = reinterpret_cast<float*>(lds + kLdsSums);
+    float* const sC = sQ + kTile;
+    unsigned long long* const sNext = reinterpret_cast<unsigned long long*>(lds + kLdsNext);
+
+    if (tid == 0) *sNext = atomicAdd(&p.counters[2], 1ull);
+    __syncthreads();
+    unsigned long long tileIdx = *sNext;
+
+    while (tileIdx < p.raster.total) {
+        unsigned tr, tc;
+        raster_decode(p.raster, tileIdx, &tr, &tc);
+        if (tr >= p.raster.tilesPerDim || tc >= p.raster.tilesPerDim) {  // padding tile of the raster
+            __syncthreads();
+            if (tid == 0) *sNext = atomicAdd(&p.counters[2], 1ull);
+            __syncthreads();
+            tileIdx = *sNext;
+            continue;
+        }
+        const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
+
+        // rows past the end of the dataset re-read the last real row; their results are masked
+        const u32x4* const gA = p.pts + (long long)rowBase * p.ld16;
+        const u32x4* const gB = p.pts + (long long)colBase * p.ld16;
+        int offA[4], offB[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = cpRow + 64 * i;
+            offA[i] = min(r, p.n - 1 - rowBase) * (int)p.ld16 + cpChunk;
+            offB[i] = min(r, p.n - 1 - colBase) * (int)p.ld16 + cpChunk;
+        }
+        if (tid < kTile) {
+            sQ[tid] = p.sums[min(rowBase + tid, p.n - 1)];
+        } else {
+            sC[tid - kTile] = p.sums[min(colBase + tid - kTile, p.n - 1)];
+        }
+
+        floatx16 acc[kFragRows][kFragCols];
+#pragma unroll
+        for (int fi = 0; fi < kFragRows; ++fi)
+#pragma unroll
+            for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[fi][fj][r] = 0.0f;
+
+        u32x4 stA[4], stB[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            stA[i] = gA[offA[i]];
+            stB[i] = gB[offB[i]];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<u32x4*>(lds + cpLds + i * 64 * kRowBytes) = stA[i];
+            *reinterpret_cast<u32x4*>(lds + kOperandBytes + cpLds + i * 64 * kRowBytes) = stB[i];
+        }
+        // reserve the next tile early so the atomic's latency hides under the k loop
+        unsigned long long nextIdx = 0;
+        if (tid == 0) nextIdx = atomicAdd(&p.counters[2], 1ull);
+        __syncthreads();
+
+        for (int s = 0; s < p.nSlabs; ++s) {
+            const bool more = s + 1 < p.nSlabs;
+            if (more) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    stA[i] = gA[offA[i] + (s + 1) * 8];
+                    stB[i] = gB[offB[i] + (s + 1) * 8];
+                }
+            }
+            const unsigned char* const buf = lds + (s & 1) * kStageBytes;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                half8 a[kFragRows], b[kFragCols];
+#pragma unroll
+                for (int fi = 0; fi < kFragRows; ++fi)
+                    a[fi] = *reinterpret_cast<const half8*>(buf + aOff[kk] + fi * 32 * kRowBytes);
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj)
+                    b[fj] = *reinterpret_cast<const half8*>(buf + bOff[kk] + fj * 32 * kRowBytes);
+#pragma unroll
+                for (int fi = 0; fi < kFragRows; ++fi)
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj)
+                        acc[fi][fj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[fi], b[fj], acc[fi][fj], 0, 0, 0);
+            }
+            if (more) {
+                unsigned char* const nb = lds + ((s + 1) & 1) * kStageBytes;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *reinterpret_cast<u32x4*>(nb + cpLds + i * 64 * kRowBytes) = stA[i];
+                    *reinterpret_cast<u32x4*>(nb + kOperandBytes + cpLds + i * 64 * kRowBytes) = stB[i];
+                }
+            }
+            __syncthreads();
+        }
+        if (tid == 0) *sNext = nextIdx;
+
+        if (kEpilogue) {
+            const int qBase = rowBase + wr * kWaveRows;
+            int cand[kFragCols];
+            float sc[kFragCols];
+#pragma unroll
+            for (int fj = 0; fj < kFragCols; ++fj) {
+                cand[fj] = colBase + wc * kWaveCols + fj * 32 + l32;
+                sc[fj] = sC[wc * kWaveCols + fj * 32 + l32];
+            }
+            unsigned mask[kFragRows];
+            const bool edge = (tr == tc) || rowBase + kTile > p.n || colBase + kTile > p.n;
+            if (edge)
+                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, hi, p.n, p.eps2, mask);
+            else
+                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, hi, p.n, p.eps2, mask);
+
+            int mine = 0;
+#pragma unroll
+            for (int fi = 0; fi < kFragRows; ++fi) mine += __builtin_popcount(mask[fi]);
+            if (__builtin_amdgcn_ballot_w64(mine != 0) != 0ull) {
+                // wave-level compaction: inclusive prefix sum of per-lane counts, one reservation
+                int incl = mine;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const int v = __shfl_up(incl, off, 64);
+                    if (lane >= off) incl += v;
+                }
+                const int total = __shfl(incl, 63, 64);
+                unsigned long long base = 0;
+                if (lane == 0) {
+                    base = atomicAdd(&p.counters[0], (unsigned long long)total);
+                    // slots past the capacity are counted but not stored (source/pair.cuh:126-132)
+                    if (base < p.cap) {
+                        const unsigned long long room = p.cap - base;
+                        atomicAdd(&p.counters[1], room < (unsigned long long)total ? room : (unsigned long long)total);
+                    }
+                }
+                base = __shfl(base, 0, 64);
+                unsigned long long slot = base + (unsigned long long)(incl - mine);
+#pragma unroll
+                for (int fi = 0; fi < kFragRows; ++fi) {
+                    unsigned m = mask[fi];
+                    while (m) {
+                        const int bit = __builtin_ctz(m);
+                        m &= m - 1;
+                        const int fj = bit >> 4, r = bit & 15;
+                        const int q = qBase + fi * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+                        if (slot < p.cap) p.pairs[slot] = make_int2(q, cand[fj]);
+                        ++slot;
+                    }
+                }
+            }
+        } else {
+            // keep the accumulators observable without spending instructions on them
+#pragma unroll
+            for (int fi = 0; fi < kFragRows; ++fi)
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj) asm volatile("" ::"v"(acc[fi][fj]));
+        }
+        if (tid == 0) atomicAdd(&p.counters[3], 1ull);
+
+        __syncthreads();
+        tileIdx = *sNext;
+    }
+}
+
+}  // namespace
+
+unsigned long long raster_count(long long n) { return make_raster(n).total; }
+
+bool raster_coord(unsigned long long idx, long long n, int* row, int* col) {
+    const Raster r = make_raster(n);
+    if (idx >= r.total) return false;
+    unsigned tr, tc;
+    raster_decode(r, idx, &tr, &tc);
+    *row = (int)tr * kTile;
+    *col = (int)tc * kTile;
+    return true;
+}
+
+hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream) {
+    const int chunksPerRow = dPad / 8;
+    int lanesPerRow = 64;
+    while (lanesPerRow > chunksPerRow) lanesPerRow >>= 1;
+    const int rowsPerWave = 64 / lanesPerRow;
+    const long long waves = ((long long)n + rowsPerWave - 1) / rowsPerWave;
+    const long long blocks = (waves + 3) / 4;
+    sum_squared_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(static_cast<const u32x4*>(points), ld / 8, n,
+                                                                        chunksPerRow, lanesPerRow, sums);
+    return hipGetLastError();
+}
+
+hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream) {
+    reset_counters_kernel<<<1, 64, 0, stream>>>(counters);
+    return hipGetLastError();
+}
+
+hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
+    static int numCUs = 0;
+    static bool configured = false;
+    if (!configured) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) return e;
+        numCUs = prop.multiProcessorCount;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&join_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&join_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    JoinParams p;
+    p.pts = static_cast<const u32x4*>(l.points);
+    p.ld16 = l.ld / 8;
+    p.n = l.n;
+    p.nSlabs = l.dPad / kSlabK;
+    p.eps2 = l.eps2;
+    p.sums = l.sums;
+    p.counters = l.counters;
+    p.pairs = static_cast<int2*>(l.pairs);
+    p.cap = l.cap;
+    p.raster = make_raster(l.n);
+    unsigned long long realTiles = (unsigned long long)p.raster.tilesPerDim * p.raster.tilesPerDim;
+    unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
+    if (grid == 0) grid = 1;
+    if (l.epilogue)
+        join_kernel<true><<<dim3(grid), dim3(kThreads), kLdsBytes, stream>>>(p);
+    else
+        join_kernel<false><<<dim3(grid), dim3(kThreads), kLdsBytes, stream>>>(p);
+    return hipGetLastError();
+}
+
+}  // namespace fasted

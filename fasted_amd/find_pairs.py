@@ -1,0 +1,172 @@
+"""ctypes binding of libfasted.so.
+
+Mirrors results/scripts/experiment/find_pairs.py of the reference: ``mmaShape`` and ``Results``
+(:24-54), ``compute_selectivity`` (:9-21), ``RerunnablePairsFinder`` (:57-89) and
+``load_findpairs`` (:93-127) keep their names, argument meaning and return types, so the
+reference's experiment drivers run unchanged on top of this module.  The raw-buffer entry
+points of include/fasted.h are bound in addition.
+"""
+import ctypes
+import os
+from typing import Callable
+
+FASTED_SORT_PAIRS = 1
+FASTED_NO_EPILOGUE = 2
+FASTED_SKIP_SUMS = 4
+
+
+def compute_selectivity(result_set_size: int, dataset_size: int) -> float:
+    """Selectivity (|R| - |D|) / |D|: mean neighbours per point with self pairs removed."""
+    return max(0, result_set_size * 1.0 - dataset_size * 1.0) / dataset_size * 1.0
+
+
+class mmaShape(ctypes.Structure):
+    _fields_ = [("m", ctypes.c_int), ("n", ctypes.c_int), ("k", ctypes.c_int)]
+
+    def __repr__(self):
+        return f"mmaShape(m={self.m}, n={self.n}, k={self.k})"
+
+
+class Results(ctypes.Structure):
+    _fields_ = [
+        ("totalTime", ctypes.c_double),
+        ("TFLOPS", ctypes.c_double),
+        ("pairsFound", ctypes.c_ulonglong),
+        ("pairsStored", ctypes.c_ulonglong),
+        ("inputProblemShape", mmaShape),
+        ("paddedProblemShape", mmaShape),
+    ]
+
+    def __repr__(self):
+        return (f"Results(totalTime={self.totalTime}, TFLOPS={self.TFLOPS}, pairsFound={self.pairsFound}, "
+                f"pairsStored={self.pairsStored}, inputProblemShape={self.inputProblemShape}, "
+                f"paddedProblemShape={self.paddedProblemShape})")
+
+    def get_selectivity(self) -> float:
+        return compute_selectivity(self.pairsFound, self.inputProblemShape.m)
+
+
+class FastedPair(ctypes.Structure):
+    _fields_ = [("QueryPoint", ctypes.c_int), ("CandidatePoint", ctypes.c_int)]
+
+
+class FastedJoinStats(ctypes.Structure):
+    _fields_ = [
+        ("sumSquaredMs", ctypes.c_float),
+        ("joinMs", ctypes.c_float),
+        ("sortMs", ctypes.c_float),
+        ("paddedN", ctypes.c_int),
+        ("paddedD", ctypes.c_int),
+        ("tiles", ctypes.c_ulonglong),
+        ("pairsFound", ctypes.c_ulonglong),
+        ("pairsStored", ctypes.c_ulonglong),
+    ]
+
+
+class RerunnablePairsFinder:
+    """Runs the full routine once, then only re-runs with a new epsilon on the resident dataset."""
+
+    def __init__(self, first_find_pairs: Callable[[float, bool], Results],
+                 rerun_find_pairs: Callable[[float, bool], Results]):
+        self._first_find_pairs = first_find_pairs
+        self._rerun_find_pairs = rerun_find_pairs
+        self._first_run = True
+
+    def __call__(self, epsilon: float, save_pairs: bool = False) -> Results:
+        if self._first_run:
+            self._first_run = False
+            return self._first_find_pairs(epsilon, save_pairs)
+        return self._rerun_find_pairs(epsilon, save_pairs)
+
+
+def library_path() -> str:
+    return os.environ.get("FASTED_LIBRARY", os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfasted.so"))
+
+
+_lib = None
+
+
+def load_findpairs(path: str = None):
+    """Loads libfasted.so and declares every entry point of include/fasted.h."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or library_path()
+    if not os.path.exists(p):
+        raise OSError(f"{p} is missing: build it with `make -C fasted_amd/csrc` (there is no CPU fallback)")
+    lib = ctypes.CDLL(p)
+    c = ctypes
+    lib.runFromExponentialDataset.restype = Results
+    lib.runFromExponentialDataset.argtypes = [c.c_int, c.c_int, c.c_double, c.c_double, c.c_double, c.c_bool]
+    lib.runFromFile.restype = Results
+    lib.runFromFile.argtypes = [c.c_char_p, c.c_double, c.c_bool]
+    lib.reRun.restype = Results
+    lib.reRun.argtypes = [c.c_double, c.c_bool]
+    lib.releaseResources.restype = None
+    lib.releaseResources.argtypes = []
+
+    lib.fasted_self_join.restype = c.c_int
+    lib.fasted_self_join.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_double, c.c_void_p, c.c_ulonglong,
+                                     c.POINTER(c.c_ulonglong), c.POINTER(c.c_ulonglong)]
+    lib.fasted_self_join_device.restype = c.c_int
+    lib.fasted_self_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_double, c.c_void_p,
+                                            c.c_void_p, c.c_ulonglong, c.c_uint, c.c_void_p,
+                                            c.POINTER(FastedJoinStats)]
+    lib.fasted_sum_squared_device.restype = c.c_int
+    lib.fasted_sum_squared_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_void_p, c.c_void_p]
+    lib.fasted_raster_coord.restype = c.c_int
+    lib.fasted_raster_coord.argtypes = [c.c_ulonglong, c.c_longlong, c.POINTER(c.c_int), c.POINTER(c.c_int)]
+    lib.fasted_raster_count.restype = c.c_ulonglong
+    lib.fasted_raster_count.argtypes = [c.c_longlong]
+    lib.fasted_resident_points.restype = c.c_void_p
+    lib.fasted_resident_points.argtypes = [c.POINTER(c.c_int)] * 4
+    lib.fasted_set_output_dir.restype = None
+    lib.fasted_set_output_dir.argtypes = [c.c_char_p]
+    lib.fasted_last_error.restype = c.c_char_p
+    lib.fasted_version.restype = c.c_char_p
+    if path is None:
+        _lib = lib
+    return lib
+
+
+class FastedError(RuntimeError):
+    pass
+
+
+def _check(lib, rc):
+    if rc != 0:
+        raise FastedError(lib.fasted_last_error().decode())
+
+
+def self_join(points_fp16, epsilon, cap=None):
+    """Host entry: (N, D) numpy float16 (or uint16 bit patterns) -> (pairs[k,2] int32 sorted, found)."""
+    import numpy as np
+
+    lib = load_findpairs()
+    a = np.ascontiguousarray(points_fp16)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    if a.dtype != np.uint16 or a.ndim != 2:
+        raise TypeError("points must be a 2-D float16 / uint16 array")
+    n, d = a.shape
+    cap = int(cap if cap is not None else n * 256)
+    out = np.empty((max(cap, 1), 2), dtype=np.int32)
+    found, stored = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+    _check(lib, lib.fasted_self_join(a.ctypes.data, n, d, float(epsilon), out.ctypes.data, cap,
+                                     ctypes.byref(found), ctypes.byref(stored)))
+    return out[:stored.value], found.value
+
+
+def self_join_device(points_ptr, n, d, ld, epsilon, pairs_ptr, cap, sums_ptr=None, flags=FASTED_SORT_PAIRS,
+                     stream=None):
+    """Device entry on raw pointers (e.g. torch ``tensor.data_ptr()``); returns FastedJoinStats."""
+    lib = load_findpairs()
+    st = FastedJoinStats()
+    _check(lib, lib.fasted_self_join_device(points_ptr, n, d, ld, float(epsilon), sums_ptr, pairs_ptr, cap, flags,
+                                            stream, ctypes.byref(st)))
+    return st
+
+
+def sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream=None):
+    lib = load_findpairs()
+    _check(lib, lib.fasted_sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream))

@@ -1,0 +1,135 @@
+/*
+ * fasted.h -- C ABI of libfasted.so, the MI355X (gfx950) epsilon self-join.
+ *
+ * Two groups of entry points:
+ *
+ *  1. The four symbols the reference's `make shared` library (main.so) exports and that
+ *     results/scripts/experiment/find_pairs.py:93-127 binds with ctypes.  Same names,
+ *     argument order, `Results` layout (returned by value) and process-global dataset
+ *     residency, so `ctypes.CDLL("libfasted.so")` can stand in for `main.so`.
+ *
+ *  2. Raw-buffer entry points ("points, N, D, epsilon in; pair list and count out") that
+ *     the reference does not have: its pairs only leave the library through a text file.
+ *     They report failure through a return code instead of exiting the process.
+ *
+ * All pointers are plain C pointers; sizes are explicit; nothing here depends on torch.
+ * The library is not re-entrant (process-global resident dataset, one device, one stream
+ * at a time), exactly like the reference (source/main.cu:33, source/findPairs.cuh:52).
+ */
+#ifndef FASTED_H
+#define FASTED_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* source/ptxMma.cuh:27-31 */
+typedef struct mmaShape {
+    int m, n, k;
+} mmaShape;
+
+/* source/findPairs.cuh:37-46; mirrored by find_pairs.py:24-44.  56 bytes. */
+typedef struct Results {
+    double totalTime;              /* seconds: upload + kernels + sort + download, no disk */
+    double TFLOPS;                 /* 2*N*N*D / (sumSquared + join kernel time) / 1e12, unpadded N, D */
+    unsigned long long pairsFound; /* every ordered pair with dist <= eps, self pairs included */
+    unsigned long long pairsStored; /* <= pairsFound when the pair buffer overflowed */
+    mmaShape inputProblemShape;    /* (N, N, D) as given */
+    mmaShape paddedProblemShape;   /* (N_pad, N_pad, D_pad) as resident on the device */
+} Results;
+
+/* source/pair.cuh:27-46.  8 bytes, ordered row-major (QueryPoint, then CandidatePoint). */
+typedef struct FastedPair {
+    int QueryPoint;
+    int CandidatePoint;
+} FastedPair;
+
+/* ---- group 1: drop-in for main.so ------------------------------------------------- */
+
+/* source/main.cu:66-67,250-261.  Seeded Exp(lambda) points rejected to [0, max], FP16. */
+Results runFromExponentialDataset(int size, int dimensionality, double lambda, double max, double epsilon,
+                                  bool savePairs);
+
+/* source/main.cu:54,263-273.  One point per line, comma separated. */
+Results runFromFile(const char* filename, double epsilon, bool savePairs);
+
+/* source/main.cu:45,275-278.  New epsilon on the dataset already resident on host+device. */
+Results reRun(double epsilon, bool savePairs);
+
+/* source/main.cu:74,280 (there it recurses into itself; here it frees the resident
+ * dataset as its comment intends, source/findPairs.cuh:766-776). */
+void releaseResources(void);
+
+/* ---- group 2: raw buffers ----------------------------------------------------------
+ * Return 0 on success, non-zero on failure; fasted_last_error() then describes it.     */
+
+typedef struct FastedJoinStats {
+    float sumSquaredMs; /* HIP-event time of the squared-norm pre-pass */
+    float joinMs;       /* HIP-event time of counter reset + join kernel */
+    float sortMs;       /* HIP-event time of the row-major sort (0 when not sorted) */
+    int paddedN;        /* rows covered by the tile grid */
+    int paddedD;        /* K extent the kernel looped over */
+    unsigned long long tiles;      /* non-empty 256x256 tiles processed */
+    unsigned long long pairsFound;
+    unsigned long long pairsStored;
+} FastedJoinStats;
+
+/* Flags for fasted_self_join_device. */
+enum {
+    FASTED_SORT_PAIRS = 1,  /* sort stored pairs row-major, as source/pair.cuh:151-158 */
+    FASTED_NO_EPILOGUE = 2, /* measurement only: run the contraction, skip test + emit */
+    FASTED_SKIP_SUMS = 4    /* d_sums already holds the squared norms */
+};
+
+/* Host buffers in, host buffers out.  `points` is N x D row-major IEEE binary16 bit
+ * patterns (what source/DataLoader/PointListBuilder.hpp:57-73 produces, before padding);
+ * up to `cap` pairs are written to `out` sorted row-major; *found counts every pair
+ * (source/pair.cuh:123-133), *stored = min(found, cap).  Replaces the body of
+ * SimSearch::FindPairs (source/findPairs.cuh:615-764) for a caller that owns its data. */
+int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon, FastedPair* out,
+                     unsigned long long cap, unsigned long long* found, unsigned long long* stored);
+
+/* Everything already in device memory (HBM-resident dataset, caller-owned pair buffer).
+ *   d_points   N rows of FP16, row stride `ld` halves (ld % 8 == 0, ld >= D rounded up to
+ *              64; the columns D..roundup(D,64) of every row must be readable zeros, or
+ *              D % 64 == 0)
+ *   d_sums     N floats of workspace/result for the squared norms (may be NULL: library
+ *              workspace is used)
+ *   d_pairs    room for `cap` pairs
+ *   stream     hipStream_t (NULL = default stream)
+ * The call synchronises the stream before returning and fills *stats.  Replaces the
+ * kernel launches of source/findPairs.cuh:632-687 (ComputeSquaredSums x2,
+ * initOnDemandRasterizer, FindPairsKernel) and the sort of :703-704. */
+int fasted_self_join_device(const void* d_points, long long n, int d, long long ld, double epsilon, float* d_sums,
+                            FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
+                            FastedJoinStats* stats);
+
+/* Squared norms only: sums[i] = sum_k x_ik^2 in FP32.  Replaces
+ * SumSqd::ComputeSquaredSums (source/sumSquared.cuh:84-118). */
+int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream);
+
+/* Tile order of the work queue: writes the (row, col) tile origin of queue index `idx`
+ * for an N_pad-row problem, or returns 0 past the end.  Host-side mirror of the device
+ * rasterizer, the counterpart of Raster::OnDemandRasterizer::nextChunk
+ * (source/rasterizer/onDemandRasterizer.cuh:78-108). */
+int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col);
+unsigned long long fasted_raster_count(long long n);
+
+/* Dataset of the last runFrom* call: padded FP16 bit patterns (host copy), for tests. */
+const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad);
+
+/* Where `savePairs` writes "<name>_<epsilon>.pairs" (default: $FASTED_PAIRS_DIR or ".").
+ * The reference hard-codes a cluster path at source/main.cu:214-215. */
+void fasted_set_output_dir(const char* dir);
+
+const char* fasted_last_error(void);
+const char* fasted_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTED_H */

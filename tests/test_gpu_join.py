@@ -1,0 +1,192 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from tests import datasets
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fasted():
+    import fasted_amd
+
+    fasted_amd.load_findpairs()
+    return fasted_amd
+
+
+def device_join(fasted, bits, eps, cap=None, flags=1, d=None, ld=None):
+    """bits: (n, ld) uint16 on host -> torch upload -> fasted_self_join_device."""
+    import torch
+
+    n = bits.shape[0]
+    ld = bits.shape[1] if ld is None else ld
+    d = ld if d is None else d
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    cap = int(cap if cap is not None else max(1024, 300 * n))
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    sums = torch.empty(n, dtype=torch.float32, device="cuda")
+    st = fasted.self_join_device(pts.data_ptr(), n, d, ld, eps, pairs.data_ptr(), cap, sums_ptr=sums.data_ptr(),
+                                 flags=flags)
+    torch.cuda.synchronize()
+    return pairs[: st.pairsStored].cpu().numpy(), st, sums.cpu().numpy()
+
+
+def check_against_fp64(bits, n, eps, got, band=1e-3):
+    rep = oracle.epsilon_band_report(bits, got, eps, n=n, band=band)
+    assert rep["outside_band"] == 0, rep
+    return rep
+
+
+@pytest.mark.parametrize("n,d", [(256, 64), (1000, 128), (4096, 128), (777, 4096), (3000, 960)])
+def test_sum_squared_matches_oracle(fasted, n, d):
+    import torch
+
+    bits = datasets.exponential(n, d, seed=n + d)
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    sums = torch.zeros(n, dtype=torch.float32, device="cuda")
+    fasted.sum_squared_device(pts.data_ptr(), n, d, d, sums.data_ptr())
+    got = sums.cpu().numpy().astype(np.float64)
+    exact = oracle.sum_squared(bits, "f64")
+    # FP32 accumulation of exact squares: relative error bounded by D * 2^-24
+    assert np.all(np.abs(got - exact) <= d * 2.0 ** -24 * exact + 1e-30)
+    # the reference's sequential round-toward-zero fold lies in the same band below the exact value
+    rz = oracle.sum_squared(bits, "rz").astype(np.float64)
+    assert np.all(np.abs(got - rz) <= 2 * d * 2.0 ** -24 * exact + 1e-30)
+
+
+def test_sum_squared_closed_form_integer_rows(fasted):
+    """Row r holds the 64 consecutive integers from 64 r (tests/python/sumSquared/sumSquared.py of
+    the reference); every partial sum is an integer below 2^24, so FP32 is exact in any order."""
+    import torch
+
+    rows, d = 32, 64
+    vals = np.arange(rows * d, dtype=np.float64).reshape(rows, d)
+    bits = oracle.quantize(vals)  # exact up to 2048
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    sums = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    fasted.sum_squared_device(pts.data_ptr(), rows, d, d, sums.data_ptr())
+    expect = np.array([sum(v * v for v in range(64 * r, 64 * r + 64)) for r in range(rows)], dtype=np.float64)
+    got = sums.cpu().numpy().astype(np.float64)
+    assert np.array_equal(got[:6], expect[:6])  # rows whose running sums stay below 2^24
+    assert np.allclose(got, expect, rtol=64 * 2.0 ** -24)
+
+
+@pytest.mark.parametrize("n,d", [(256, 64), (512, 128), (300, 64), (1025, 192), (2048, 1024)])
+def test_integer_points_exact_pair_set(fasted, n, d):
+    """Integer coordinates make every dot product exact, so the pair set must equal the FP64
+    join bit for bit (epsilon^2 sits between two integers: no pair is near the threshold)."""
+    bits = datasets.small_integers(n, d, high=3, seed=7 * n + d)
+    x = bits.view(np.float16).astype(np.float64)
+    d2 = ((x[:64, None, :] - x[None, :64, :]) ** 2).sum(-1)
+    target = np.sort(d2[np.triu_indices(64, 1)])[40]
+    eps = float(np.sqrt(target + 0.5))
+    got, st, _ = device_join(fasted, bits, eps)
+    truth = oracle.self_join_f64(bits, eps)
+    assert st.pairsFound == len(truth) and st.pairsStored == len(truth)
+    assert np.array_equal(got, truth)
+
+
+def test_identity_points(fasted):
+    """Unit vectors e_i (the reference's GenerateIdentityMatrixPoints fixture, main.cu:113-131):
+    distinct points are sqrt(2) apart, duplicates are at distance 0."""
+    n, d = 512, 256
+    x = np.zeros((n, d), dtype=np.float16)
+    x[np.arange(n), np.arange(n) % d] = 1.0
+    bits = x.view(np.uint16)
+    got, st, _ = device_join(fasted, bits, 1.0)
+    expect = np.array([(i, j) for i in range(n) for j in range(n) if i % d == j % d], dtype=np.int32)
+    assert np.array_equal(got, expect)
+    got, st, _ = device_join(fasted, bits, 1.5)
+    assert st.pairsFound == n * n
+
+
+def test_plumbing_config_full_fp64_check(fasted):
+    """N=4096 x D=128 Exp(40) clipped to [0,1], ~32 neighbours/point, entire pair set vs FP64."""
+    n, d = 4096, 128
+    bits = datasets.exponential(n, d, seed=2024)
+    eps = datasets.epsilon_for_neighbours(bits, 32)
+    got, st, _ = device_join(fasted, bits, eps)
+    rep = check_against_fp64(bits, n, eps, got)
+    sel = (st.pairsFound - n) / n
+    assert 20 < sel < 50, sel
+    assert rep["both"] >= rep["truth_total"] - rep["band_pairs"]
+    print("plumbing config:", rep, "selectivity", sel)
+    # the reference's own arithmetic model (RZ norms, FP32 dot) agrees up to the same band
+    model = oracle.self_join_f32(bits, eps)
+    check_against_fp64(bits, n, eps, model)
+
+
+@pytest.mark.parametrize("n,d", [(1, 64), (2, 64), (255, 64), (257, 128), (1000, 320), (5000, 64)])
+def test_ragged_sizes(fasted, n, d):
+    bits = datasets.uniform_bytes(n, d, seed=n)
+    eps = datasets.epsilon_for_neighbours(bits, min(8, max(n - 1, 0) / 2)) if n > 2 else 0.5
+    got, st, _ = device_join(fasted, bits, eps)
+    check_against_fp64(bits, n, eps, got)
+    assert st.pairsFound >= n  # every self pair is reported
+    assert set(map(tuple, got[got[:, 0] == got[:, 1]])) == {(i, i) for i in range(n)}
+
+
+def test_dimension_padding_through_host_entry(fasted):
+    """D not a multiple of 64 goes through the host entry, which zero-pads on upload."""
+    n, d = 700, 100
+    bits = datasets.uniform_bytes(n, d, seed=5)
+    eps = datasets.epsilon_for_neighbours(bits, 10)
+    got, found = fasted.self_join(bits, eps)
+    assert found == len(got)
+    check_against_fp64(bits, n, eps, got)
+
+
+def test_tiny_epsilon_reports_exactly_the_self_pairs(fasted):
+    """eps = 0.001 on the seeded Exp(40) data finds exactly N pairs (the self pairs), the count the
+    reference's ExpoDataSpeedVsSize_OnDemandRasterizer.json holds for D in {64,128,256}."""
+    lib = fasted.load_findpairs()
+    for n, d in [(1000, 64), (2154, 128), (1000, 256)]:
+        r = lib.runFromExponentialDataset(n, d, 40.0, 10.0, 0.001, False)
+        assert r.pairsFound == n and r.pairsStored == n
+        assert (r.inputProblemShape.m, r.inputProblemShape.n, r.inputProblemShape.k) == (n, n, d)
+        assert r.paddedProblemShape.k % 64 == 0 and r.paddedProblemShape.m % 256 == 0
+    lib.releaseResources()
+
+
+def test_pair_buffer_overflow_is_soft(fasted):
+    """found keeps counting, stored stops at the capacity, nothing is written past it
+    (source/pair.cuh:123-133)."""
+    import torch
+
+    n, d = 1024, 64
+    bits = datasets.uniform_bytes(n, d, seed=3)
+    eps = datasets.epsilon_for_neighbours(bits, 20)
+    full, st_full, _ = device_join(fasted, bits, eps)
+    cap = 1000
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    buf = torch.full((cap + 64, 2), -7, dtype=torch.int32, device="cuda")
+    st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, buf.data_ptr(), cap, flags=0)
+    assert st.pairsFound == st_full.pairsFound
+    assert st.pairsStored == cap
+    host = buf.cpu().numpy()
+    assert (host[cap:] == -7).all()
+    stored = {tuple(p) for p in host[:cap]}
+    assert len(stored) == cap and stored <= {tuple(p) for p in full}
+
+
+def test_rerun_changes_epsilon_on_resident_data(fasted):
+    lib = fasted.load_findpairs()
+    n, d = 3000, 128
+    r0 = lib.runFromExponentialDataset(n, d, 40.0, 10.0, 0.3, False)
+    np_, dp_, npad, dpad = (ctypes.c_int() for _ in range(4))
+    ptr = lib.fasted_resident_points(ctypes.byref(np_), ctypes.byref(dp_), ctypes.byref(npad), ctypes.byref(dpad))
+    bits = np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_uint16)), (npad.value, dpad.value)).copy()
+    assert (np_.value, dp_.value) == (n, d)
+    assert np.array_equal(bits[:n, :d], oracle.quantize(oracle.exponential_points(n, d, 40.0, 10.0)))
+    truth0 = oracle.self_join_f64(bits, 0.3, n=n)
+    r1 = lib.reRun(0.33, False)
+    truth1 = oracle.self_join_f64(bits, 0.33, n=n)
+    assert abs(int(r0.pairsFound) - len(truth0)) <= max(4, len(truth0) // 1000)
+    assert abs(int(r1.pairsFound) - len(truth1)) <= max(4, len(truth1) // 1000)
+    assert r1.pairsFound > r0.pairsFound
+    assert r0.TFLOPS > 0 and r0.totalTime > 0
+    lib.releaseResources()
