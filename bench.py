@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the epsilon self-join hot path on one MI355X.
+
+One "step" is one pass of the hot path over the resident dataset: squared-norm pre-pass,
+queue/counter reset and the fused MFMA join kernel (the reference's TFLOPS window,
+source/findPairs.cuh:625-697,729,745-747).  Inputs are generated on the device and are
+resident in HBM before the timed region starts.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3]
+
+prints ONE JSON line: metric = self-join TFLOPS (2*N^2*D / time), plus `roofline`
+(the join kernel against the dense FP16 MFMA peak) and `cpu_baseline` (the FP64 brute-force
+checker timed on this box's host cores on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2516.6  # MI355X dense FP16 MFMA: 256 CU x 4 SIMD x 1024 FLOP/clk x 2.4 GHz
+
+CONFIGS = {
+    # name: (N, D, generator, mean neighbours, label)
+    "c1": (4096, 128, "exponential", 32, "plumbing 4096x128 Exp(40)"),
+    "c2": (100_000, 128, "uniform_bytes", 64, "low-dim 100000x128 U{0..255}/255"),
+    "c3": (1_000_000, 4096, "exponential", 16, "headline 1000000x4096 Exp(40)"),
+    "c4": (500_000, 960, "gaussian_mixture", 100, "clustered 500000x960 GMM(1000, sigma=0.05)"),
+    "c5": (2_000_000, 384, "unit_normal", 1000, "output-heavy 2000000x384 unit-normalised N(0,1)"),
+}
+
+
+def generate_points(torch, kind, n, d, seed):
+    """FP16 dataset generated on the device in row chunks (seeded)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    out = torch.empty((n, d), dtype=torch.float16, device="cuda")
+    rows = max(1, min(n, (1 << 28) // d))
+    centers = None
+    if kind == "gaussian_mixture":
+        centers = torch.rand((1000, d), generator=g, device="cuda", dtype=torch.float32)
+    for r0 in range(0, n, rows):
+        r1 = min(n, r0 + rows)
+        m = r1 - r0
+        if kind == "exponential":
+            x = torch.empty((m, d), device="cuda", dtype=torch.float32).exponential_(40.0, generator=g).clamp_(0.0, 1.0)
+        elif kind == "uniform_bytes":
+            x = torch.randint(0, 256, (m, d), generator=g, device="cuda").to(torch.float32) / 255.0
+        elif kind == "gaussian_mixture":
+            which = torch.randint(0, 1000, (m,), generator=g, device="cuda")
+            x = centers[which] + 0.05 * torch.randn((m, d), generator=g, device="cuda", dtype=torch.float32)
+        elif kind == "unit_normal":
+            x = torch.randn((m, d), generator=g, device="cuda", dtype=torch.float32)
+            x = x / x.norm(dim=1, keepdim=True)
+        else:
+            raise ValueError(kind)
+        out[r0:r1] = x.to(torch.float16)
+        del x
+    return out
+
+
+def calibrate_epsilon(torch, pts, neighbours, sample=256, seed=4242):
+    """epsilon from a seeded sample of query rows: the distance quantile that yields the wanted
+    mean number of neighbours per point (self pairs excluded).  Harness code (torch FP32)."""
+    n, d = pts.shape
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    m = min(sample, n)
+    rows = torch.randperm(n, generator=g, device="cuda")[:m]
+    q = pts[rows].to(torch.float32)
+    qs = (q * q).sum(1)
+    k = int(round(neighbours * m)) + m + 1  # + the m self pairs
+    best = torch.full((0,), float("inf"), device="cuda")
+    chunk = max(1, min(n, (1 << 27) // d))
+    for c0 in range(0, n, chunk):
+        c = pts[c0:c0 + chunk].to(torch.float32)
+        d2 = qs[:, None] + (c * c).sum(1)[None, :] - 2.0 * (q @ c.T)
+        flat = d2.reshape(-1)
+        kk = min(k, flat.numel())
+        best = torch.cat([best, torch.topk(flat, kk, largest=False).values])
+        if best.numel() > k:
+            best = torch.topk(best, k, largest=False).values
+        del c, d2, flat
+    best = torch.sort(best).values.clamp_min(0.0)
+    want = int(round(neighbours * m)) + m  # self pairs sit at (about) zero
+    want = min(want, best.numel() - 1)
+    eps2 = 0.5 * (best[want - 1] + best[want]).item()
+    return math.sqrt(eps2)
+
+
+def cpu_baseline(torch, pts, eps, budget_s=15.0):
+    """FP64 brute-force join (the CPU checker) on a bounded sample: Q query rows against the
+    first Nc points of the same dataset, on this box's host cores."""
+    import numpy as np
+
+    import oracle
+
+    n, d = pts.shape
+    nc = int(min(n, max(1024, (1 << 27) // d)))
+    host = pts[:nc].cpu().numpy().view(np.uint16)
+    cores = min(oracle.num_threads(), 16)
+    os.environ["OMP_NUM_THREADS"] = str(cores)
+
+    def run(q):
+        t0 = time.perf_counter()
+        pairs = oracle.self_join_f64(host, eps, n=nc, rows=(0, q))
+        return time.perf_counter() - t0, len(pairs)
+
+    q = min(nc, max(cores * 4, 64))
+    t, _ = run(q)
+    q2 = int(min(nc, max(q, q * budget_s / max(t, 1e-3))))
+    if q2 > q:
+        t, _ = run(q2)
+        q = q2
+    tflops = 2.0 * q * nc * d / t / 1e12
+    return {
+        "value": tflops, "unit": "TFLOPS", "cores": cores, "kind": "port",
+        "sample": f"{q} query rows x first {nc} points x D={d}, FP64, {t:.2f} s "
+                  f"(full-size extrapolation: {2.0 * n * n * d / (tflops * 1e12):.0f} s)",
+    }
+
+
+def load_traffic(name):
+    """HBM bytes per join-kernel launch measured with rocprofv3 --pmc (committed under profiles/)."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name)
+    except OSError:
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
+    ap.add_argument("--n", type=int, default=0, help="override the number of points")
+    ap.add_argument("--d", type=int, default=0, help="override the dimensionality")
+    ap.add_argument("--eps", type=float, default=0.0, help="skip calibration and use this epsilon")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-epilogue", action="store_true", help="measurement: contraction only")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU hot path only: run with --gpus 1 (no multi-GPU path exists)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import fasted_amd
+    from fasted_amd import find_pairs as fp
+
+    if not torch.cuda.is_available():
+        print("no GPU visible: the join has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    fasted_amd.load_findpairs()
+
+    n, d, kind, neighbours, label = CONFIGS[args.config]
+    n = args.n or n
+    d = args.d or d
+    if args.n or args.d:
+        label = f"{kind} {n}x{d} (override of {args.config})"
+    pts = generate_points(torch, kind, n, d, seed=20260 + n % 997)
+    eps = args.eps or calibrate_epsilon(torch, pts, neighbours)
+    cap = int(min(n * 256, max(n * (neighbours + 1) * 2, 1 << 20)))
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    sums = torch.empty(n, dtype=torch.float32, device="cuda")
+    flags = fp.FASTED_NO_EPILOGUE if args.no_epilogue else 0
+
+    def step():
+        return fp.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, sums_ptr=sums.data_ptr(),
+                                   flags=flags)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    stats = [step() for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_per_step = wall * 1000.0 / args.steps
+    flops = 2.0 * n * n * d
+    tflops = flops / (ms_per_step / 1000.0) / 1e12
+    st = stats[-1]
+    join_ms = sum(s.joinMs for s in stats) / len(stats)
+    sums_ms = sum(s.sumSquaredMs for s in stats) / len(stats)
+    achieved = flops / (join_ms / 1000.0) / 1e12
+    out = {
+        "metric": "self-join TFLOPS (2*N^2*D/s)", "value": tflops, "unit": "TFLOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": label, "N": n, "D": d, "epsilon": eps, "mean_neighbours_target": neighbours,
+                   "pairs_found": int(st.pairsFound), "pairs_stored": int(st.pairsStored),
+                   "mean_neighbours": (st.pairsFound - n) / n, "pairs_per_s": st.pairsFound / (ms_per_step / 1000.0),
+                   "pct_of_fp16_peak": 100.0 * tflops / PEAK_FP16_TFLOPS, "tiles": int(st.tiles),
+                   "sum_squared_ms": sums_ms, "join_kernel_ms": join_ms, "epilogue": not args.no_epilogue},
+        "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
+                     "traffic": load_traffic(args.config if not (args.n or args.d) else "")},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
