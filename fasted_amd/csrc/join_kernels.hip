@@ -147,13 +147,17 @@ __device__ __forceinline__ void test_block(const floatx16 (&acc)[kFragRows][kFra
 template <bool kEpilogue>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
     const int wr = wave >> 2, wc = wave & 3;
     const int l32 = lane & 31, hi = lane >> 5;
 
-    // copy role: 8 consecutive lanes fetch one 128-byte row segment of a slab
-    const int cpRow = tid >> 3, cpChunk = tid & 7;
-    const int cpLds = cpRow * kRowBytes + ((cpChunk ^ swz(cpRow)) << 4);  // rows +64*i keep swz
+    // copy role: global -> LDS without passing through registers (global_load_lds_dwordx4).
+    // One wave instruction fills 1 KiB of LDS = 8 rows of a slab, lane l landing in row l/8,
+    // chunk slot l%8; the swizzle is applied on the global side by choosing which 16-byte
+    // chunk of the row each lane fetches, so the 8 lanes of a row still read one 128-byte line.
+    // Wave w owns rows [32w, 32w+32) of both operands: 4 instructions each.
+    const int cpRow0 = wave * 32 + (lane >> 3);
 
     // fragment role: lane reads row l32 of a 32-row block, chunk 2*kk + hi
     int aOff[4], bOff[4];
@@ -190,9 +194,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         int offA[4], offB[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int r = cpRow + 64 * i;
-            offA[i] = min(r, p.n - 1 - rowBase) * (int)p.ld16 + cpChunk;
-            offB[i] = min(r, p.n - 1 - colBase) * (int)p.ld16 + cpChunk;
+            const int r = cpRow0 + 8 * i;
+            const int chunk = (lane & 7) ^ swz(r);
+            offA[i] = min(r, p.n - 1 - rowBase) * (int)p.ld16 + chunk;
+            offB[i] = min(r, p.n - 1 - colBase) * (int)p.ld16 + chunk;
         }
         if (tid < kTile) {
             sQ[tid] = p.sums[min(rowBase + tid, p.n - 1)];
@@ -208,54 +213,55 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[fi][fj][r] = 0.0f;
 
-        u32x4 stA[4], stB[4];
+        auto issue_slab = [&](int slab, int stage) {
+            unsigned char* const dst = lds + stage * kStageBytes + wave * 32 * kRowBytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            stA[i] = gA[offA[i]];
-            stB[i] = gB[offB[i]];
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4*>(lds + cpLds + i * 64 * kRowBytes) = stA[i];
-            *reinterpret_cast<u32x4*>(lds + kOperandBytes + cpLds + i * 64 * kRowBytes) = stB[i];
-        }
+            for (int i = 0; i < 4; ++i) {
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gA + offA[i] + slab * 8),
+                                                 (__attribute__((address_space(3))) void*)(dst + i * 8 * kRowBytes), 16,
+                                                 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gB + offB[i] + slab * 8),
+                                                 (__attribute__((address_space(3))) void*)(dst + kOperandBytes +
+                                                                                           i * 8 * kRowBytes),
+                                                 16, 0, 0);
+            }
+        };
+        issue_slab(0, 0);
         // reserve the next tile early so the atomic's latency hides under the k loop
         unsigned long long nextIdx = 0;
         if (tid == 0) nextIdx = atomicAdd(&p.counters[2], 1ull);
         __syncthreads();
 
         for (int s = 0; s < p.nSlabs; ++s) {
-            const bool more = s + 1 < p.nSlabs;
-            if (more) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    stA[i] = gA[offA[i] + (s + 1) * 8];
-                    stB[i] = gB[offB[i] + (s + 1) * 8];
-                }
-            }
+            if (s + 1 < p.nSlabs) issue_slab(s + 1, (s + 1) & 1);
             const unsigned char* const buf = lds + (s & 1) * kStageBytes;
+            half8 a[2][kFragRows], b[2][kFragCols];
+#pragma unroll
+            for (int fi = 0; fi < kFragRows; ++fi)
+                a[0][fi] = *reinterpret_cast<const half8*>(buf + aOff[0] + fi * 32 * kRowBytes);
+#pragma unroll
+            for (int fj = 0; fj < kFragCols; ++fj)
+                b[0][fj] = *reinterpret_cast<const half8*>(buf + bOff[0] + fj * 32 * kRowBytes);
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                half8 a[kFragRows], b[kFragCols];
+                const int cur = kk & 1, nxt = cur ^ 1;
+                if (kk + 1 < 4) {
 #pragma unroll
-                for (int fi = 0; fi < kFragRows; ++fi)
-                    a[fi] = *reinterpret_cast<const half8*>(buf + aOff[kk] + fi * 32 * kRowBytes);
+                    for (int fi = 0; fi < kFragRows; ++fi)
+                        a[nxt][fi] = *reinterpret_cast<const half8*>(buf + aOff[kk + 1] + fi * 32 * kRowBytes);
 #pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj)
-                    b[fj] = *reinterpret_cast<const half8*>(buf + bOff[kk] + fj * 32 * kRowBytes);
+                    for (int fj = 0; fj < kFragCols; ++fj)
+                        b[nxt][fj] = *reinterpret_cast<const half8*>(buf + bOff[kk + 1] + fj * 32 * kRowBytes);
+                }
+                // keep the next k-step's LDS reads in flight under this k-step's MFMAs
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fi = 0; fi < kFragRows; ++fi)
 #pragma unroll
                     for (int fj = 0; fj < kFragCols; ++fj)
-                        acc[fi][fj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[fi], b[fj], acc[fi][fj], 0, 0, 0);
-            }
-            if (more) {
-                unsigned char* const nb = lds + ((s + 1) & 1) * kStageBytes;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    *reinterpret_cast<u32x4*>(nb + cpLds + i * 64 * kRowBytes) = stA[i];
-                    *reinterpret_cast<u32x4*>(nb + kOperandBytes + cpLds + i * 64 * kRowBytes) = stB[i];
-                }
+                        acc[fi][fj] =
+                            __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][fi], b[cur][fj], acc[fi][fj], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
             __syncthreads();
         }
