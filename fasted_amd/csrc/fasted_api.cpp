@@ -58,7 +58,7 @@ struct Workspace {
     size_t sumsCap = 0;
 
     void ensure(size_t n) {
-        if (!counters) HIP_CHECK(hipMalloc(&counters, 4 * sizeof(unsigned long long)));
+        if (!counters) HIP_CHECK(hipMalloc(&counters, fasted::counter_words() * sizeof(unsigned long long)));
         if (n > sumsCap) {
             if (sums) HIP_CHECK(hipFree(sums));
             sums = nullptr;
@@ -149,7 +149,7 @@ void join_on_device(const void* dPoints, long long n, int d, long long ld, doubl
         stats->sortMs = sortMs;
         stats->paddedN = round_up(n, fasted::kTile);
         stats->paddedD = dPad;
-        stats->tiles = c[3];
+        stats->tiles = c[2];
         stats->pairsFound = c[0];
         stats->pairsStored = c[1];
     }
@@ -385,7 +385,7 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
 
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     if (n < 1 || !row || !col) return 0;
-    return fasted::raster_coord(idx, n, row, col) ? 1 : 0;
+    return fasted::raster_coord(idx, n, row, col);
 }
 
 unsigned long long fasted_raster_count(long long n) { return n < 1 ? 0ull : fasted::raster_count(n); }

@@ -17,7 +17,7 @@ struct JoinLaunch {
     int dPad;                    // K extent, multiple of kSlabK
     float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
     const float* sums;           // squared norms
-    unsigned long long* counters;  // [0] found, [1] stored, [2] queue head, [3] tiles done
+    unsigned long long* counters;  // counter_words() words: [0] found, [1] stored, [2] tiles done, queue heads
     void* pairs;                 // FastedPair[cap]
     unsigned long long cap;
     bool epilogue;               // false: contraction only (measurement)
@@ -25,7 +25,8 @@ struct JoinLaunch {
 
 // Host mirror of the device tile order.
 unsigned long long raster_count(long long n);
-bool raster_coord(unsigned long long idx, long long n, int* row, int* col);
+int raster_coord(unsigned long long idx, long long n, int* row, int* col);
+int counter_words();
 
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream);
 hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream);

@@ -41,30 +41,43 @@ constexpr int kFragRows = kWaveRows / 32, kFragCols = kWaveCols / 32;  // 4 x 2 
 // 16 consecutive rows at one logical chunk cover all 64 four-byte banks exactly once.
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// Work queues.  The N x N matrix of 256x256 tiles is cut into super-squares of 16 x 16 tiles;
+// a super-square is cut into 8 sub-rectangles of 4 x 8 tiles, one per XCD (accelerator die).
+// Each XCD has its own queue head: its t-th pop is tile (t % 32) of its sub-rectangle of
+// super-square t / 32.  The 32 workgroups resident on one XCD therefore work on 4 query panels
+// and 8 candidate panels at a time and share them through that XCD's L2, and all 8 XCDs stay
+// inside one super-square (16 + 16 panels) that the Infinity Cache holds.  An XCD whose queue
+// is exhausted steals from the next XCD's queue, so the tail stays balanced.
 struct Raster {
     unsigned tilesPerDim;
     unsigned squaresPerDim;
-    unsigned long long total;
+    unsigned long long perQueue;  // pops each queue serves
 };
+
+constexpr int kQueues = 8;                 // one per XCD
+constexpr int kSubRows = 4, kSubCols = 8;  // sub-rectangle of one XCD inside a super-square
+constexpr int kSubTiles = kSubRows * kSubCols;
+static_assert(kRaster == 16 && kSubTiles * kQueues == kRaster * kRaster, "8 sub-rectangles tile a super-square");
+constexpr int kCounterFound = 0, kCounterStored = 1, kCounterTiles = 2;
+constexpr int kQueueBase = 16, kQueueStride = 16;  // queue heads sit on separate 128-byte lines
+constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
 __host__ __device__ inline Raster make_raster(long long n) {
     Raster r;
     r.tilesPerDim = (unsigned)((n + kTile - 1) / kTile);
     r.squaresPerDim = (r.tilesPerDim + kRaster - 1) / kRaster;
-    r.total = (unsigned long long)r.squaresPerDim * r.squaresPerDim * (kRaster * kRaster);
+    r.perQueue = (unsigned long long)r.squaresPerDim * r.squaresPerDim * kSubTiles;
     return r;
 }
 
-// Queue index -> tile (row, col) in tile units.  Indices are dealt out in kRaster x kRaster
-// squares (row-major over squares, row-major inside) so that workgroups running at the same
-// time share query and candidate panels in L2 / Infinity Cache.  Tiles outside the
-// tilesPerDim grid are padding: the caller skips them.
-__host__ __device__ inline void raster_decode(const Raster& r, unsigned long long idx, unsigned* tr, unsigned* tc) {
-    const unsigned area = kRaster * kRaster;
-    unsigned long long sq = idx / area;
-    unsigned local = (unsigned)(idx % area);
-    *tr = (unsigned)(sq / r.squaresPerDim) * kRaster + local / kRaster;
-    *tc = (unsigned)(sq % r.squaresPerDim) * kRaster + local % kRaster;
+// Pop t of queue q -> tile (row, col) in tile units.  Tiles outside the tilesPerDim grid are
+// padding of the last super-squares: the caller skips them.
+__host__ __device__ inline void raster_decode(const Raster& r, unsigned q, unsigned long long t, unsigned* tr,
+                                              unsigned* tc) {
+    const unsigned long long sq = t / kSubTiles;
+    const unsigned local = (unsigned)(t % kSubTiles);
+    *tr = (unsigned)(sq / r.squaresPerDim) * kRaster + (q >> 1) * kSubRows + local / kSubCols;
+    *tc = (unsigned)(sq % r.squaresPerDim) * kRaster + (q & 1) * kSubCols + local % kSubCols;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -94,7 +107,7 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
 }
 
 __global__ void reset_counters_kernel(unsigned long long* c) {
-    if (threadIdx.x < 4) c[threadIdx.x] = 0ull;
+    if (threadIdx.x < kCounterWords) c[threadIdx.x] = 0ull;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -172,18 +185,35 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     float* const sC = sQ + kTile;
     unsigned long long* const sNext = reinterpret_cast<unsigned long long*>(lds + kLdsNext);
 
-    if (tid == 0) *sNext = atomicAdd(&p.counters[2], 1ull);
-    __syncthreads();
-    unsigned long long tileIdx = *sNext;
+    // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
+    const unsigned home = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (kQueues - 1);
 
-    while (tileIdx < p.raster.total) {
+    // A ticket is queue * perQueue + position; kDone means every queue is exhausted.
+    const unsigned long long kDone = ~0ull;
+    auto take = [&](unsigned firstQueue, unsigned long long firstPos) -> unsigned long long {
+        // firstPos was already popped from firstQueue; on exhaustion move on to the other queues
+        unsigned q = firstQueue;
+        unsigned long long pos = firstPos;
+        for (int tries = 0; tries < kQueues; ++tries) {
+            if (pos < p.raster.perQueue) return (unsigned long long)q * p.raster.perQueue + pos;
+            q = (q + 1) & (kQueues - 1);
+            if (tries + 1 < kQueues) pos = atomicAdd(&p.counters[kQueueBase + q * kQueueStride], 1ull);
+        }
+        return kDone;
+    };
+
+    if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
+    __syncthreads();
+    unsigned long long ticket = *sNext;
+
+    while (ticket != kDone) {
         unsigned tr, tc;
-        raster_decode(p.raster, tileIdx, &tr, &tc);
+        raster_decode(p.raster, (unsigned)(ticket / p.raster.perQueue), ticket % p.raster.perQueue, &tr, &tc);
         if (tr >= p.raster.tilesPerDim || tc >= p.raster.tilesPerDim) {  // padding tile of the raster
             __syncthreads();
-            if (tid == 0) *sNext = atomicAdd(&p.counters[2], 1ull);
+            if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
             __syncthreads();
-            tileIdx = *sNext;
+            ticket = *sNext;
             continue;
         }
         const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
@@ -228,8 +258,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         };
         issue_slab(0, 0);
         // reserve the next tile early so the atomic's latency hides under the k loop
-        unsigned long long nextIdx = 0;
-        if (tid == 0) nextIdx = atomicAdd(&p.counters[2], 1ull);
+        unsigned long long nextPos = 0;
+        if (tid == 0) nextPos = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         __syncthreads();
 
         for (int s = 0; s < p.nSlabs; ++s) {
@@ -265,7 +295,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             }
             __syncthreads();
         }
-        if (tid == 0) *sNext = nextIdx;
+        if (tid == 0) *sNext = take(home, nextPos);
 
         if (kEpilogue) {
             const int qBase = rowBase + wr * kWaveRows;
@@ -297,11 +327,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 const int total = __shfl(incl, 63, 64);
                 unsigned long long base = 0;
                 if (lane == 0) {
-                    base = atomicAdd(&p.counters[0], (unsigned long long)total);
+                    base = atomicAdd(&p.counters[kCounterFound], (unsigned long long)total);
                     // slots past the capacity are counted but not stored (source/pair.cuh:126-132)
                     if (base < p.cap) {
                         const unsigned long long room = p.cap - base;
-                        atomicAdd(&p.counters[1], room < (unsigned long long)total ? room : (unsigned long long)total);
+                        atomicAdd(&p.counters[kCounterStored], room < (unsigned long long)total ? room : (unsigned long long)total);
                     }
                 }
                 base = __shfl(base, 0, 64);
@@ -326,26 +356,31 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) asm volatile("" ::"v"(acc[fi][fj]));
         }
-        if (tid == 0) atomicAdd(&p.counters[3], 1ull);
+        if (tid == 0) atomicAdd(&p.counters[kCounterTiles], 1ull);
 
         __syncthreads();
-        tileIdx = *sNext;
+        ticket = *sNext;
     }
 }
 
 }  // namespace
 
-unsigned long long raster_count(long long n) { return make_raster(n).total; }
+unsigned long long raster_count(long long n) { return make_raster(n).perQueue * kQueues; }
 
-bool raster_coord(unsigned long long idx, long long n, int* row, int* col) {
+// Index idx enumerates the queues round-robin: queue idx % 8, position idx / 8 -- the order in
+// which eight equally fast XCDs would take the tiles.  Returns 0 past the end, 2 for a padding
+// tile that the kernel skips, 1 for a real tile.
+int raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     const Raster r = make_raster(n);
-    if (idx >= r.total) return false;
+    if (idx >= r.perQueue * kQueues) return 0;
     unsigned tr, tc;
-    raster_decode(r, idx, &tr, &tc);
+    raster_decode(r, (unsigned)(idx % kQueues), idx / kQueues, &tr, &tc);
     *row = (int)tr * kTile;
     *col = (int)tc * kTile;
-    return true;
+    return (tr < r.tilesPerDim && tc < r.tilesPerDim) ? 1 : 2;
 }
+
+int counter_words() { return kCounterWords; }
 
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream) {
     const int chunksPerRow = dPad / 8;
@@ -360,7 +395,7 @@ hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad,
 }
 
 hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream) {
-    reset_counters_kernel<<<1, 64, 0, stream>>>(counters);
+    reset_counters_kernel<<<1, 256, 0, stream>>>(counters);
     return hipGetLastError();
 }
 
