@@ -18,11 +18,12 @@
 // candidate tile are staged in LDS in the same [256 rows][64 halves] form.
 #include "join_kernels.h"
 
+#include <type_traits>
+
 namespace fasted {
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -34,7 +35,7 @@ constexpr int kLdsSums = 2 * kStageBytes;           // s_q[256] then s_c[256]
 constexpr int kLdsNext = kLdsSums + 2 * kTile * 4;  // next queue index
 constexpr int kLdsBytes = kLdsNext + 16;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
-constexpr int kFragRows = kWaveRows / 32, kFragCols = kWaveCols / 32;  // 4 x 2 MFMA 32x32 blocks
+constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
 // 16-byte chunk c of LDS row r lives at chunk slot c ^ swz(r).  Any 8 consecutive rows hit
 // 8 distinct slots, and rows r, r+8 differ in the low slot bit while sharing row parity, so
@@ -124,36 +125,37 @@ struct JoinParams {
     Raster raster;
 };
 
-// Distance test of one wave's 128x64 block.  kEdge: the tile touches the diagonal or the
+// Distance test of one wave's 128x64 block of accumulators.  acc[fi][fj] is a 16x16 MFMA block:
+// lane l holds column l%16 and rows 4*(l/16) .. +3.  kEdge: the tile touches the diagonal or the
 // ragged end of the dataset, so self pairs are forced and padded rows/cols are masked
-// (source/warpMma.cuh:257-259).  Returns per-lane hit bits: mask[fi] bit (fj*16 + r).
+// (source/warpMma.cuh:257-259).  Returns per-lane hit bits: mask[fi/2] bit ((fi&1)*16 + fj*4 + r).
 template <bool kEdge>
-__device__ __forceinline__ void test_block(const floatx16 (&acc)[kFragRows][kFragCols], const float* sQ,
+__device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const float* sQ,
                                            const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
-                                           int hi, int n, float eps2, unsigned (&mask)[kFragRows]) {
+                                           int quad, int n, float eps2, unsigned (&mask)[kFragRows / 2]) {
 #pragma unroll
-    for (int fi = 0; fi < kFragRows; ++fi) {
+    for (int fp = 0; fp < kFragRows / 2; ++fp) {
         unsigned m = 0;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const floatx4 sq = *reinterpret_cast<const floatx4*>(sQ + fi * 32 + g * 8 + hi * 4);
+        for (int h = 0; h < 2; ++h) {
+            const int fi = fp * 2 + h;
+            const floatx4 sq = *reinterpret_cast<const floatx4*>(sQ + fi * 16 + quad * 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int r = g * 4 + e;
+            for (int fj = 0; fj < kFragCols; ++fj) {
 #pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) {
+                for (int r = 0; r < 4; ++r) {
                     // (s_q + s_c) - 2*acc, FP32, as source/warpMma.cuh:241-242
-                    const float d2 = (sq[e] + sc[fj]) - (2.0f * acc[fi][fj][r]);
+                    const float d2 = (sq[r] + sc[fj]) - (2.0f * acc[fi][fj][r]);
                     bool hit = d2 <= eps2;
                     if (kEdge) {
-                        const int q = qBase + fi * 32 + g * 8 + hi * 4 + e;
+                        const int q = qBase + fi * 16 + quad * 4 + r;
                         hit = (hit || q == cand[fj]) && q < n && cand[fj] < n;
                     }
-                    m |= (hit ? 1u : 0u) << (fj * 16 + r);
+                    m = hit ? (m | (1u << (h * 16 + fj * 4 + r))) : m;
                 }
             }
         }
-        mask[fi] = m;
+        mask[fp] = m;
     }
 }
 
@@ -163,7 +165,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
     const int wr = wave >> 2, wc = wave & 3;
-    const int l32 = lane & 31, hi = lane >> 5;
+    const int l16 = lane & 15, quad = lane >> 4;
 
     // copy role: global -> LDS without passing through registers (global_load_lds_dwordx4).
     // One wave instruction fills 1 KiB of LDS = 8 rows of a slab, lane l landing in row l/8,
@@ -172,13 +174,14 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // Wave w owns rows [32w, 32w+32) of both operands: 4 instructions each.
     const int cpRow0 = wave * 32 + (lane >> 3);
 
-    // fragment role: lane reads row l32 of a 32-row block, chunk 2*kk + hi
-    int aOff[4], bOff[4];
+    // fragment role (v_mfma_f32_16x16x32_f16): lane reads row l%16 of a 16-row block and the
+    // 8 halves k = 8*(l/16) .. +7 of a 32-wide k-step, i.e. chunk 4*ks + l/16 of the slab row.
+    int aOff[2], bOff[2];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-        const int slot = ((kk * 2 + hi) ^ swz(l32)) << 4;
-        aOff[kk] = (wr * kWaveRows + l32) * kRowBytes + slot;
-        bOff[kk] = kOperandBytes + (wc * kWaveCols + l32) * kRowBytes + slot;
+    for (int ks = 0; ks < 2; ++ks) {
+        const int slot = ((ks * 4 + quad) ^ swz(l16)) << 4;
+        aOff[ks] = (wr * kWaveRows + l16) * kRowBytes + slot;
+        bOff[ks] = kOperandBytes + (wc * kWaveCols + l16) * kRowBytes + slot;
     }
 
     float* const sQ = reinterpret_cast<float*>(lds + kLdsSums);
@@ -219,15 +222,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
 
         // rows past the end of the dataset re-read the last real row; their results are masked
-        const u32x4* const gA = p.pts + (long long)rowBase * p.ld16;
-        const u32x4* const gB = p.pts + (long long)colBase * p.ld16;
-        int offA[4], offB[4];
+        const char* const gA = reinterpret_cast<const char*>(p.pts + (long long)rowBase * p.ld16);
+        const char* const gB = reinterpret_cast<const char*>(p.pts + (long long)colBase * p.ld16);
+        unsigned offA[4], offB[4];  // byte offsets from the tile's first row
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = cpRow0 + 8 * i;
             const int chunk = (lane & 7) ^ swz(r);
-            offA[i] = min(r, p.n - 1 - rowBase) * (int)p.ld16 + chunk;
-            offB[i] = min(r, p.n - 1 - colBase) * (int)p.ld16 + chunk;
+            offA[i] = (unsigned)(min(r, p.n - 1 - rowBase) * (int)p.ld16 + chunk) * 16u;
+            offB[i] = (unsigned)(min(r, p.n - 1 - colBase) * (int)p.ld16 + chunk) * 16u;
         }
         if (tid < kTile) {
             sQ[tid] = p.sums[min(rowBase + tid, p.n - 1)];
@@ -235,66 +238,85 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             sC[tid - kTile] = p.sums[min(colBase + tid - kTile, p.n - 1)];
         }
 
-        floatx16 acc[kFragRows][kFragCols];
+        floatx4 acc[kFragRows][kFragCols];
 #pragma unroll
         for (int fi = 0; fi < kFragRows; ++fi)
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[fi][fj][r] = 0.0f;
+                for (int r = 0; r < 4; ++r) acc[fi][fj][r] = 0.0f;
 
-        auto issue_slab = [&](int slab, int stage) {
-            unsigned char* const dst = lds + stage * kStageBytes + wave * 32 * kRowBytes;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gA + offA[i] + slab * 8),
-                                                 (__attribute__((address_space(3))) void*)(dst + i * 8 * kRowBytes), 16,
-                                                 0, 0);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gB + offB[i] + slab * 8),
-                                                 (__attribute__((address_space(3))) void*)(dst + kOperandBytes +
-                                                                                           i * 8 * kRowBytes),
-                                                 16, 0, 0);
-            }
+        // One 1-KiB global->LDS transfer of this wave: j = 0..7 alternates query / candidate rows.
+        auto issue_load = [&](unsigned slabByte, int stage, int j) {
+            const int i = j >> 1;
+            unsigned char* const dst = lds + stage * kStageBytes + (j & 1) * kOperandBytes +
+                                       (wave * 32 + i * 8) * kRowBytes;
+            // uniform 64-bit base + 32-bit lane offset (formed here so it stays a 32-bit add)
+            const char* const src = (j & 1) ? gB + (offB[i] + slabByte) : gA + (offA[i] + slabByte);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
         };
-        issue_slab(0, 0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) issue_load(0u, 0, j);
         // reserve the next tile early so the atomic's latency hides under the k loop
         unsigned long long nextPos = 0;
         if (tid == 0) nextPos = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         __syncthreads();
 
-        for (int s = 0; s < p.nSlabs; ++s) {
-            if (s + 1 < p.nSlabs) issue_slab(s + 1, (s + 1) & 1);
+        // One slab = 2 k-steps of 32; a k-step is two halves of 16 MFMAs (query blocks 0-3, then
+        // 4-7, each against the 4 candidate blocks).  The instruction order is pinned with
+        // scheduling barriers: the LDS reads for the next half are issued ahead of the MFMAs of
+        // the current half, and the 8 global->LDS transfers of the next slab are spread one per
+        // 8 MFMAs, so neither the LDS nor the texture-address queue makes a wave wait with the
+        // matrix pipe idle.
+        auto slab_step = [&](int s, auto prefetch) {
+            constexpr bool kPrefetch = decltype(prefetch)::value;
+            const unsigned nextByte = (unsigned)(s + 1) * kRowBytes;
             const unsigned char* const buf = lds + (s & 1) * kStageBytes;
-            half8 a[2][kFragRows], b[2][kFragCols];
-#pragma unroll
-            for (int fi = 0; fi < kFragRows; ++fi)
-                a[0][fi] = *reinterpret_cast<const half8*>(buf + aOff[0] + fi * 32 * kRowBytes);
+            half8 aLo[4], aHi[4], b[2][kFragCols];
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
-                b[0][fj] = *reinterpret_cast<const half8*>(buf + bOff[0] + fj * 32 * kRowBytes);
+                b[0][fj] = *reinterpret_cast<const half8*>(buf + bOff[0] + fj * 16 * kRowBytes);
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const int cur = kk & 1, nxt = cur ^ 1;
-                if (kk + 1 < 4) {
+            for (int fi = 0; fi < 4; ++fi)
+                aLo[fi] = *reinterpret_cast<const half8*>(buf + aOff[0] + fi * 16 * kRowBytes);
 #pragma unroll
-                    for (int fi = 0; fi < kFragRows; ++fi)
-                        a[nxt][fi] = *reinterpret_cast<const half8*>(buf + aOff[kk + 1] + fi * 32 * kRowBytes);
+            for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-                    for (int fj = 0; fj < kFragCols; ++fj)
-                        b[nxt][fj] = *reinterpret_cast<const half8*>(buf + bOff[kk + 1] + fj * 32 * kRowBytes);
-                }
-                // keep the next k-step's LDS reads in flight under this k-step's MFMAs
+                for (int fi = 0; fi < 4; ++fi)
+                    aHi[fi] = *reinterpret_cast<const half8*>(buf + aOff[ks] + (fi + 4) * 16 * kRowBytes);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int fi = 0; fi < kFragRows; ++fi)
+                for (int fj = 0; fj < kFragCols; ++fj) {
+                    if (kPrefetch && (fj & 1) == 0) issue_load(nextByte, (s + 1) & 1, ks * 4 + (fj >> 1));
+#pragma unroll
+                    for (int fi = 0; fi < 4; ++fi)
+                        acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (ks == 0) {
 #pragma unroll
                     for (int fj = 0; fj < kFragCols; ++fj)
-                        acc[fi][fj] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][fi], b[cur][fj], acc[fi][fj], 0, 0, 0);
+                        b[1][fj] = *reinterpret_cast<const half8*>(buf + bOff[1] + fj * 16 * kRowBytes);
+#pragma unroll
+                    for (int fi = 0; fi < 4; ++fi)
+                        aLo[fi] = *reinterpret_cast<const half8*>(buf + aOff[1] + fi * 16 * kRowBytes);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj) {
+                    if (kPrefetch && (fj & 1) == 0) issue_load(nextByte, (s + 1) & 1, ks * 4 + 2 + (fj >> 1));
+#pragma unroll
+                    for (int fi = 0; fi < 4; ++fi)
+                        acc[fi + 4][fj] =
+                            __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             __syncthreads();
-        }
+        };
+        for (int s = 0; s + 1 < p.nSlabs; ++s) slab_step(s, std::true_type{});
+        slab_step(p.nSlabs - 1, std::false_type{});
         if (tid == 0) *sNext = take(home, nextPos);
 
         if (kEpilogue) {
@@ -303,19 +325,19 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             float sc[kFragCols];
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj) {
-                cand[fj] = colBase + wc * kWaveCols + fj * 32 + l32;
-                sc[fj] = sC[wc * kWaveCols + fj * 32 + l32];
+                cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
+                sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
             }
-            unsigned mask[kFragRows];
+            unsigned mask[kFragRows / 2];
             const bool edge = (tr == tc) || rowBase + kTile > p.n || colBase + kTile > p.n;
             if (edge)
-                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, hi, p.n, p.eps2, mask);
+                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
             else
-                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, hi, p.n, p.eps2, mask);
+                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
 
             int mine = 0;
 #pragma unroll
-            for (int fi = 0; fi < kFragRows; ++fi) mine += __builtin_popcount(mask[fi]);
+            for (int fp = 0; fp < kFragRows / 2; ++fp) mine += __builtin_popcount(mask[fp]);
             if (__builtin_amdgcn_ballot_w64(mine != 0) != 0ull) {
                 // wave-level compaction: inclusive prefix sum of per-lane counts, one reservation
                 int incl = mine;
@@ -331,20 +353,22 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                     // slots past the capacity are counted but not stored (source/pair.cuh:126-132)
                     if (base < p.cap) {
                         const unsigned long long room = p.cap - base;
-                        atomicAdd(&p.counters[kCounterStored], room < (unsigned long long)total ? room : (unsigned long long)total);
+                        atomicAdd(&p.counters[kCounterStored],
+                                  room < (unsigned long long)total ? room : (unsigned long long)total);
                     }
                 }
                 base = __shfl(base, 0, 64);
                 unsigned long long slot = base + (unsigned long long)(incl - mine);
 #pragma unroll
-                for (int fi = 0; fi < kFragRows; ++fi) {
-                    unsigned m = mask[fi];
+                for (int fp = 0; fp < kFragRows / 2; ++fp) {
+                    unsigned m = mask[fp];
                     while (m) {
                         const int bit = __builtin_ctz(m);
                         m &= m - 1;
-                        const int fj = bit >> 4, r = bit & 15;
-                        const int q = qBase + fi * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-                        if (slot < p.cap) p.pairs[slot] = make_int2(q, cand[fj]);
+                        const int fi = fp * 2 + (bit >> 4), fj = (bit >> 2) & 3, r = bit & 3;
+                        const int q = qBase + fi * 16 + quad * 4 + r;
+                        const int c = colBase + wc * kWaveCols + fj * 16 + l16;
+                        if (slot < p.cap) p.pairs[slot] = make_int2(q, c);
                         ++slot;
                     }
                 }
