@@ -33,7 +33,8 @@ constexpr int kOperandBytes = kTile * kRowBytes;    // 32 KiB per operand per st
 constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 64 KiB
 constexpr int kLdsSums = 2 * kStageBytes;           // s_q[256] then s_c[256]
 constexpr int kLdsNext = kLdsSums + 2 * kTile * 4;  // next queue index
-constexpr int kLdsBytes = kLdsNext + 16;
+constexpr int kLdsWaveMax = kLdsNext + 16;          // per-wave max of the tile's squared norms
+constexpr int kLdsBytes = kLdsWaveMax + 8 * 4;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
@@ -187,6 +188,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     float* const sQ = reinterpret_cast<float*>(lds + kLdsSums);
     float* const sC = sQ + kTile;
     unsigned long long* const sNext = reinterpret_cast<unsigned long long*>(lds + kLdsNext);
+    float* const sWaveMax = reinterpret_cast<float*>(lds + kLdsWaveMax);
 
     // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
     const unsigned home = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (kQueues - 1);
@@ -232,10 +234,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             offA[i] = (unsigned)(min(r, p.n - 1 - rowBase) * (int)p.ld16 + chunk) * 16u;
             offB[i] = (unsigned)(min(r, p.n - 1 - colBase) * (int)p.ld16 + chunk) * 16u;
         }
-        if (tid < kTile) {
-            sQ[tid] = p.sums[min(rowBase + tid, p.n - 1)];
-        } else {
-            sC[tid - kTile] = p.sums[min(colBase + tid - kTile, p.n - 1)];
+        {
+            // squared norms of the tile's 256 queries and 256 candidates, plus their maximum
+            // (it scales the safety margin of the epilogue's screening test)
+            const float mySum = tid < kTile ? p.sums[min(rowBase + tid, p.n - 1)]
+                                            : p.sums[min(colBase + tid - kTile, p.n - 1)];
+            sQ[tid] = mySum;  // sC == sQ + kTile
+            float m = __builtin_fabsf(mySum);
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, off, 64));
+            if (lane == 0) sWaveMax[wave] = m;
         }
 
         floatx4 acc[kFragRows][kFragCols];
@@ -328,12 +336,46 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
                 sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
             }
-            unsigned mask[kFragRows / 2];
+            // Screening pass (1.5 VALU ops per element): in real arithmetic a hit is
+            //   acc - s_q/2 >= (s_c - eps^2)/2,
+            // so take the per-column maximum of acc - s_q/2 and compare it, with a margin that
+            // covers every FP32 rounding of both forms, against the column's right-hand side.
+            // Only waves with a candidate run the exact reference formula below; on tiles that
+            // touch the diagonal or the ragged end every wave does.
             const bool edge = (tr == tc) || rowBase + kTile > p.n || colBase + kTile > p.n;
-            if (edge)
-                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
-            else
-                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
+            bool candidate = edge;
+            if (!edge) {
+                float sMax = sWaveMax[0];
+#pragma unroll
+                for (int w = 1; w < 8; ++w) sMax = __builtin_fmaxf(sMax, sWaveMax[w]);
+                const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
+                float best[kFragCols];
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj) best[fj] = -__builtin_inff();
+#pragma unroll
+                for (int fi = 0; fi < kFragRows; ++fi) {
+                    const floatx4 hq = *reinterpret_cast<const floatx4*>(sQ + wr * kWaveRows + fi * 16 + quad * 4) * 0.5f;
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj) {
+                        const floatx4 f = acc[fi][fj] - hq;
+                        best[fj] = __builtin_fmaxf(best[fj], __builtin_fmaxf(__builtin_fmaxf(f[0], f[1]),
+                                                                             __builtin_fmaxf(f[2], f[3])));
+                    }
+                }
+                bool any = false;
+#pragma unroll
+                for (int fj = 0; fj < kFragCols; ++fj) any = any || (best[fj] >= 0.5f * (sc[fj] - p.eps2) - margin);
+                candidate = __builtin_amdgcn_ballot_w64(any) != 0ull;
+            }
+            unsigned mask[kFragRows / 2];
+#pragma unroll
+            for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
+            if (candidate) {
+                if (edge)
+                    test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
+                else
+                    test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
+            }
 
             int mine = 0;
 #pragma unroll
