@@ -63,7 +63,7 @@ def generate_points(torch, kind, n, d, seed):
     return out
 
 
-def calibrate_epsilon(torch, pts, neighbours, sample=256, seed=4242):
+def calibrate_epsilon(torch, pts, neighbours, sample=1024, seed=4242):
     """epsilon from a seeded sample of query rows: the distance quantile that yields the wanted
     mean number of neighbours per point (self pairs excluded).  Harness code (torch FP32)."""
     n, d = pts.shape
@@ -168,7 +168,8 @@ def main():
         label = f"{kind} {n}x{d} (override of {args.config})"
     pts = generate_points(torch, kind, n, d, seed=20260 + n % 997)
     eps = args.eps or calibrate_epsilon(torch, pts, neighbours)
-    cap = int(min(n * 256, max(n * (neighbours + 1) * 2, 1 << 20)))
+    # pair buffer: the reference's N*256 records, or 1.25x the expected count when that is larger
+    cap = int(max(n * 256, 1.25 * n * (neighbours + 1)))
     pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
     sums = torch.empty(n, dtype=torch.float32, device="cuda")
     flags = fp.FASTED_NO_EPILOGUE if args.no_epilogue else 0

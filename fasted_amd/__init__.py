@@ -14,6 +14,7 @@ from .find_pairs import (  # noqa: F401
     library_path,
     load_findpairs,
     mmaShape,
+    resident_points,
     self_join,
     self_join_device,
     sum_squared_device,
@@ -21,5 +22,5 @@ from .find_pairs import (  # noqa: F401
 
 __all__ = [
     "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "library_path",
-    "load_findpairs", "mmaShape", "self_join", "self_join_device", "sum_squared_device",
+    "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_device", "sum_squared_device",
 ]

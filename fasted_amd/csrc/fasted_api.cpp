@@ -383,6 +383,24 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
     });
 }
 
+int fasted_load_exponential_dataset(int size, int dimensionality, double lambda, double max) {
+    return guarded([&] {
+        fasted::ExponentialSource src(size, dimensionality, lambda, max);
+        g_res.drop_device();
+        g_res.table = fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+    });
+}
+
+int fasted_load_file(const char* filename) {
+    return guarded([&] {
+        fasted::CsvSource src(std::string(filename ? filename : ""), ',');
+        g_res.drop_device();
+        g_res.table = fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+    });
+}
+
+const char* fasted_resident_name(void) { return g_res.table.name.c_str(); }
+
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     if (n < 1 || !row || !col) return 0;
     return fasted::raster_coord(idx, n, row, col);

@@ -118,6 +118,11 @@ def load_findpairs(path: str = None):
     lib.fasted_raster_coord.argtypes = [c.c_ulonglong, c.c_longlong, c.POINTER(c.c_int), c.POINTER(c.c_int)]
     lib.fasted_raster_count.restype = c.c_ulonglong
     lib.fasted_raster_count.argtypes = [c.c_longlong]
+    lib.fasted_load_exponential_dataset.restype = c.c_int
+    lib.fasted_load_exponential_dataset.argtypes = [c.c_int, c.c_int, c.c_double, c.c_double]
+    lib.fasted_load_file.restype = c.c_int
+    lib.fasted_load_file.argtypes = [c.c_char_p]
+    lib.fasted_resident_name.restype = c.c_char_p
     lib.fasted_resident_points.restype = c.c_void_p
     lib.fasted_resident_points.argtypes = [c.POINTER(c.c_int)] * 4
     lib.fasted_set_output_dir.restype = None
@@ -165,6 +170,19 @@ def self_join_device(points_ptr, n, d, ld, epsilon, pairs_ptr, cap, sums_ptr=Non
     _check(lib, lib.fasted_self_join_device(points_ptr, n, d, ld, float(epsilon), sums_ptr, pairs_ptr, cap, flags,
                                             stream, ctypes.byref(st)))
     return st
+
+
+def resident_points():
+    """Host copy of the resident dataset: (bits[n_pad, d_pad] uint16, n, d, name)."""
+    import numpy as np
+
+    lib = load_findpairs()
+    n, d, n_pad, d_pad = (ctypes.c_int() for _ in range(4))
+    ptr = lib.fasted_resident_points(ctypes.byref(n), ctypes.byref(d), ctypes.byref(n_pad), ctypes.byref(d_pad))
+    if not ptr:
+        return None
+    arr = np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_uint16)), (n_pad.value, d_pad.value))
+    return arr.copy(), n.value, d.value, lib.fasted_resident_name().decode()
 
 
 def sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream=None):

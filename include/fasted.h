@@ -112,15 +112,27 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
  * SumSqd::ComputeSquaredSums (source/sumSquared.cuh:84-118). */
 int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream);
 
-/* Tile order of the work queue: writes the (row, col) tile origin of queue index `idx`
- * for an N_pad-row problem, or returns 0 past the end.  Host-side mirror of the device
- * rasterizer, the counterpart of Raster::OnDemandRasterizer::nextChunk
+/* Tile order of the work queues: writes the (row, col) origin, in points, of the 256x256 tile
+ * that queue index `idx` stands for in an n-point problem.  idx enumerates the eight per-XCD
+ * queues round-robin (queue idx % 8, position idx / 8).  Returns 0 past the end, 1 for a real
+ * tile, 2 for a padding tile of the last raster squares (the kernel skips those).  Host-side
+ * mirror of the device rasterizer, the counterpart of Raster::OnDemandRasterizer::nextChunk
  * (source/rasterizer/onDemandRasterizer.cuh:78-108). */
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col);
 unsigned long long fasted_raster_count(long long n);
 
-/* Dataset of the last runFrom* call: padded FP16 bit patterns (host copy), for tests. */
+/* Build the resident host dataset only (no GPU work): what runFromExponentialDataset /
+ * runFromFile do before the join (source/main.cu:205-208), so that reRun() can follow.
+ * Counterparts of ExponentialPointGenerator + PointListBuilder::build
+ * (source/DataLoader/ExponentialPointGenerator.hpp:35-57, PointListBuilder.hpp:132-192) and
+ * FilePointGenerator (source/DataLoader/FilePointGenerator.hpp:33-56). */
+int fasted_load_exponential_dataset(int size, int dimensionality, double lambda, double max);
+int fasted_load_file(const char* filename);
+
+/* Resident dataset: padded FP16 bit patterns (host copy) and its name
+ * (PointGenerator::getName, source/DataLoader/PointGenerator.hpp:27-30). */
 const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad);
+const char* fasted_resident_name(void);
 
 /* Where `savePairs` writes "<name>_<epsilon>.pairs" (default: $FASTED_PAIRS_DIR or ".").
  * The reference hard-codes a cluster path at source/main.cu:214-215. */

@@ -1,0 +1,181 @@
+"""CPU-side tests of the shipped library: every symbol of include/fasted.h is exported, the
+`Results` layout matches the reference's ctypes mirror, the host data path reproduces the
+reference's datasets, and the host mirror of the tile queues covers every tile exactly once.
+No compute entry point is called here (there is no GPU and no CPU fallback)."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+import fasted_amd
+import oracle
+from fasted_amd import find_pairs as fp
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+GOLDEN = json.load(open(os.path.join(GOLDEN_DIR, "reference_loader.json")))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return fasted_amd.load_findpairs()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "fasted.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{]*\)\s*;", text)
+    return sorted(set(names))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_functions()
+    assert {"runFromExponentialDataset", "runFromFile", "reRun", "releaseResources", "fasted_self_join",
+            "fasted_self_join_device", "fasted_sum_squared_device"} <= set(names)
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/fasted.h but not exported"
+
+
+def test_results_layout_matches_the_reference_mirror():
+    # results/scripts/experiment/find_pairs.py:24-44 of the reference: 56 bytes, same offsets
+    assert ctypes.sizeof(fp.mmaShape) == 12
+    assert ctypes.sizeof(fp.Results) == 56
+    offs = {n: getattr(fp.Results, n).offset for n, _ in fp.Results._fields_}
+    assert offs == {"totalTime": 0, "TFLOPS": 8, "pairsFound": 16, "pairsStored": 24, "inputProblemShape": 32,
+                    "paddedProblemShape": 44}
+    assert ctypes.sizeof(fp.FastedPair) == 8
+    assert lib_signature_ok()
+
+
+def lib_signature_ok():
+    lib = fasted_amd.load_findpairs()
+    return (lib.runFromExponentialDataset.restype is fp.Results and lib.reRun.restype is fp.Results
+            and lib.runFromFile.argtypes == [ctypes.c_char_p, ctypes.c_double, ctypes.c_bool])
+
+
+def test_selectivity_and_rerunnable_finder_follow_the_reference():
+    assert fp.compute_selectivity(300, 100) == 2.0
+    assert fp.compute_selectivity(50, 100) == 0.0  # never negative
+    r = fp.Results(pairsFound=1100, inputProblemShape=fp.mmaShape(100, 100, 8))
+    assert r.get_selectivity() == 10.0
+    calls = []
+    finder = fp.RerunnablePairsFinder(lambda e, s: calls.append(("first", e, s)) or "A",
+                                      lambda e, s: calls.append(("rerun", e, s)) or "B")
+    assert [finder(0.1), finder(0.2, True), finder(0.3)] == ["A", "B", "B"]
+    assert calls == [("first", 0.1, False), ("rerun", 0.2, True), ("rerun", 0.3, False)]
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(OSError):
+        fasted_amd.load_findpairs(str(tmp_path / "nope.so"))
+
+
+# ---------------------------------------------------------------- host data path
+@pytest.mark.parametrize("case", GOLDEN["exponential"], ids=lambda c: c["name"])
+def test_exponential_dataset_equals_reference_golden(lib, case):
+    assert lib.fasted_load_exponential_dataset(case["n"], case["d"], case["lambda"], case["max"]) == 0
+    bits, n, d, name = fasted_amd.resident_points()
+    assert (n, d, name) == (case["n"], case["d"], case["name"])
+    assert bits.shape[1] == case["d_pad"] and bits.shape[0] % 256 == 0 and bits.shape[0] >= n
+    assert np.array_equal(bits[:n, :d], np.array(case["bits"], dtype=np.uint16))
+    assert bits[n:].sum() == 0 and bits[:, d:].sum() == 0
+
+
+def test_exponential_dataset_equals_oracle_on_a_larger_case(lib):
+    assert lib.fasted_load_exponential_dataset(700, 200, 40.0, 10.0) == 0
+    bits, n, d, _ = fasted_amd.resident_points()
+    assert np.array_equal(bits[:n, :d], oracle.quantize(oracle.exponential_points(700, 200, 40.0, 10.0)))
+
+
+def test_csv_dataset_equals_reference_golden(lib):
+    g = GOLDEN["csv"]
+    assert lib.fasted_load_file(os.path.join(GOLDEN_DIR, g["file"]).encode()) == 0
+    bits, n, d, name = fasted_amd.resident_points()
+    assert (n, d, name, bits.shape[1]) == (g["n"], g["d"], g["name"], g["d_pad"])
+    assert np.array_equal(bits[:n, :d], np.array(g["bits"], dtype=np.uint16))
+    # the same values through the checker's quantiser
+    vals = np.loadtxt(os.path.join(GOLDEN_DIR, g["file"]), delimiter=",")
+    with np.errstate(over="ignore"):
+        assert np.array_equal(bits[:n, :d], oracle.quantize(vals))
+
+
+def test_csv_error_paths(lib, tmp_path):
+    assert lib.fasted_load_file(str(tmp_path / "missing.csv").encode()) != 0
+    assert b"Failed to open file" in lib.fasted_last_error()
+    ragged = tmp_path / "ragged.csv"
+    ragged.write_text("1,2,3\n4,5\n")
+    assert lib.fasted_load_file(str(ragged).encode()) != 0
+    assert lib.fasted_last_error().decode() == GOLDEN["ragged_error"]
+    empty = tmp_path / "empty.csv"
+    empty.write_text("")
+    assert lib.fasted_load_file(str(empty).encode()) != 0
+    assert lib.fasted_last_error().decode() == GOLDEN["empty_error"]
+    bad = tmp_path / "bad.csv"
+    bad.write_text("1,2\n3,x\n")
+    assert lib.fasted_load_file(str(bad).encode()) != 0
+    trailing = tmp_path / "trail.csv"
+    trailing.write_text("0.5,0.25,\n1,2,\n")  # a trailing delimiter adds no field
+    assert lib.fasted_load_file(str(trailing).encode()) == 0
+    _, n, d, name = fasted_amd.resident_points()
+    assert (n, d, name) == (2, 2, "trail")
+
+
+def test_raw_entry_rejects_bad_arguments_without_touching_a_gpu(lib):
+    found, stored = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+    assert lib.fasted_self_join(None, 10, 8, 0.1, None, 0, ctypes.byref(found), ctypes.byref(stored)) != 0
+    assert b"null" in lib.fasted_last_error()
+    st = fp.FastedJoinStats()
+    assert lib.fasted_self_join_device(None, 10, 64, 64, 0.1, None, None, 0, 0, None, ctypes.byref(st)) != 0
+    buf = (ctypes.c_uint16 * 64)()
+    for n, d, ld in [(0, 64, 64), (10, 0, 64), (10, 64, 60), (10, 100, 64)]:
+        rc = lib.fasted_self_join_device(ctypes.addressof(buf), n, d, ld, 0.1, None, None, 0, 0, None, ctypes.byref(st))
+        assert rc != 0 and lib.fasted_last_error()
+
+
+# ---------------------------------------------------------------- tile queues (host mirror)
+@pytest.mark.parametrize("n", [1, 256, 257, 4096, 5000, 100_000])
+def test_tile_queues_cover_every_tile_exactly_once(lib, n):
+    tiles = -(-n // 256)
+    total = lib.fasted_raster_count(n)
+    assert total % (8 * 32) == 0 and total >= tiles * tiles
+    row, col = ctypes.c_int(), ctypes.c_int()
+    seen = np.zeros((tiles, tiles), dtype=np.int32)
+    padding = 0
+    step = 1 if total <= 300_000 else None
+    idxs = range(total) if step else None
+    for idx in idxs:
+        kind = lib.fasted_raster_coord(idx, n, ctypes.byref(row), ctypes.byref(col))
+        assert kind in (1, 2)
+        assert row.value % 256 == 0 and col.value % 256 == 0
+        if kind == 1:
+            seen[row.value // 256, col.value // 256] += 1
+        else:
+            padding += 1
+            assert row.value >= n or col.value >= n
+    assert (seen == 1).all()
+    assert padding == total - tiles * tiles
+    assert lib.fasted_raster_coord(total, n, ctypes.byref(row), ctypes.byref(col)) == 0
+
+
+def test_tile_queue_locality(lib):
+    """32 consecutive positions of one queue are one 4 x 8 block of tiles (one XCD's share of a
+    16 x 16 super-square), and the 8 queues together tile that super-square."""
+    n = 256 * 48
+    row, col = ctypes.c_int(), ctypes.c_int()
+    for square in (0, 1, 4):
+        cover = set()
+        for q in range(8):
+            block = []
+            for t in range(32):
+                idx = (square * 32 + t) * 8 + q
+                assert lib.fasted_raster_coord(idx, n, ctypes.byref(row), ctypes.byref(col)) == 1
+                block.append((row.value // 256, col.value // 256))
+            r0, c0 = block[0]
+            assert block == [(r0 + t // 8, c0 + t % 8) for t in range(32)]
+            cover |= set(block)
+        rs, cs = min(r for r, _ in cover), min(c for _, c in cover)
+        assert cover == {(rs + i, cs + j) for i in range(16) for j in range(16)}
+        assert rs % 16 == 0 and cs % 16 == 0
