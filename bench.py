@@ -145,6 +145,8 @@ def main():
     ap.add_argument("--eps", type=float, default=0.0, help="skip calibration and use this epsilon")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogue", action="store_true", help="measurement: contraction only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 1 GiB read + 1 GiB write elementwise kernel (to scale FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU hot path only: run with --gpus 1 (no multi-GPU path exists)",
@@ -160,6 +162,15 @@ def main():
         print("no GPU visible: the join has no CPU fallback", file=sys.stderr)
         sys.exit(1)
     fasted_amd.load_findpairs()
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            torch.mul(src, 1.0, out=dst)  # one kernel: reads 2^30 bytes, writes 2^30 bytes
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy": {"read_bytes": 1 << 30, "write_bytes": 1 << 30, "launches": 4}}))
+        return
 
     n, d, kind, neighbours, label = CONFIGS[args.config]
     n = args.n or n
@@ -196,13 +207,14 @@ def main():
     out = {
         "metric": "self-join TFLOPS (2*N^2*D/s)", "value": tflops, "unit": "TFLOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": label, "N": n, "D": d, "epsilon": eps, "mean_neighbours_target": neighbours,
                    "pairs_found": int(st.pairsFound), "pairs_stored": int(st.pairsStored),
                    "mean_neighbours": (st.pairsFound - n) / n, "pairs_per_s": st.pairsFound / (ms_per_step / 1000.0),
                    "pct_of_fp16_peak": 100.0 * tflops / PEAK_FP16_TFLOPS, "tiles": int(st.tiles),
-                   "sum_squared_ms": sums_ms, "join_kernel_ms": join_ms, "epilogue": not args.no_epilogue},
+                   "sum_squared_ms": sums_ms, "join_kernel_ms": join_ms, "epilogue": not args.no_epilogue,
+                   "accumulate": "f32", "peak_used_tflops": PEAK_FP16_TFLOPS},
         "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": load_traffic(args.config if not (args.n or args.d) else "")},

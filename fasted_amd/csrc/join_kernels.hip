@@ -38,10 +38,14 @@ constexpr int kLdsBytes = kLdsWaveMax + 8 * 4;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
-// 16-byte chunk c of LDS row r lives at chunk slot c ^ swz(r).  Any 8 consecutive rows hit
-// 8 distinct slots, and rows r, r+8 differ in the low slot bit while sharing row parity, so
-// 16 consecutive rows at one logical chunk cover all 64 four-byte banks exactly once.
-__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+// 16-byte chunk c of LDS row r lives at chunk slot c ^ swz(r).  A row is 128 B, so row parity
+// picks the half of the 64 four-byte banks and the slot picks 4 banks inside it.  gfx950 serves
+// a ds_read_b128 in four phases of 16 lanes -- {0-3,12-15,20-23,24-27}, {4-7,8-11,16-19,28-31}
+// and the same two groups +32 -- and the fragment read of v_mfma_f32_16x16x32_f16 has lane l on
+// row l%16, chunk 4*ks + l/16.  With swz(r) = (r>>1)&7 every phase touches 16 distinct
+// (parity, slot) pairs, i.e. all 64 banks once: no bank conflict (checked exhaustively on the
+// host by tests, and with the SQ_LDS_BANK_CONFLICT counter on the device).
+__host__ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 // Work queues.  The N x N matrix of 256x256 tiles is cut into super-squares of 16 x 16 tiles;
 // a super-square is cut into 8 sub-rectangles of 4 x 8 tiles, one per XCD (accelerator die).
