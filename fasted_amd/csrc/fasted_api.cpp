@@ -406,6 +406,8 @@ int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col)
     return fasted::raster_coord(idx, n, row, col);
 }
 
+int fasted_lds_chunk_slot(int row, int chunk) { return fasted::lds_chunk_slot(row, chunk); }
+
 unsigned long long fasted_raster_count(long long n) { return n < 1 ? 0ull : fasted::raster_count(n); }
 
 const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad) {

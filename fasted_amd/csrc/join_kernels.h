@@ -27,6 +27,8 @@ struct JoinLaunch {
 unsigned long long raster_count(long long n);
 int raster_coord(unsigned long long idx, long long n, int* row, int* col);
 int counter_words();
+// Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).
+int lds_chunk_slot(int row, int chunk);
 
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream);
 hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream);

@@ -452,6 +452,8 @@ int raster_coord(unsigned long long idx, long long n, int* row, int* col) {
 
 int counter_words() { return kCounterWords; }
 
+int lds_chunk_slot(int row, int chunk) { return (chunk ^ swz(row)) & 7; }
+
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream) {
     const int chunksPerRow = dPad / 8;
     int lanesPerRow = 64;

@@ -121,6 +121,12 @@ int fasted_sum_squared_device(const void* d_points, long long n, int d, long lon
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col);
 unsigned long long fasted_raster_count(long long n);
 
+/* LDS placement of the kernel's operand tiles: the 16-byte chunk `chunk` (0..7) of row `row` of a
+ * 64-wide k-slab is stored at the returned slot (0..7) of that row's 128 bytes.  Host mirror of the
+ * device swizzle, the counterpart of SimSearch::SwizzleAddress (source/findPairs.cuh:161-166); exported
+ * so that its bank-conflict freedom can be checked without a GPU. */
+int fasted_lds_chunk_slot(int row, int chunk);
+
 /* Build the resident host dataset only (no GPU work): what runFromExponentialDataset /
  * runFromFile do before the join (source/main.cu:205-208), so that reRun() can follow.
  * Counterparts of ExponentialPointGenerator + PointListBuilder::build
