@@ -63,7 +63,7 @@ def generate_points(torch, kind, n, d, seed):
     return out
 
 
-def calibrate_epsilon(torch, pts, neighbours, sample=1024, seed=4242):
+def calibrate_epsilon(torch, pts, neighbours, sample=4096, seed=4242):
     """epsilon from a seeded sample of query rows: the distance quantile that yields the wanted
     mean number of neighbours per point (self pairs excluded).  Harness code (torch FP32)."""
     n, d = pts.shape

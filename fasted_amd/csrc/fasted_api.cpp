@@ -135,8 +135,12 @@ void join_on_device(const void* dPoints, long long n, int d, long long ld, doubl
     HIP_CHECK(hipEventRecord(t.ev[2], stream));
     HIP_CHECK(hipStreamSynchronize(stream));
 
+    // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
+    // counted only (source/pair.cuh:123-133), so stored = min(found, capacity)
     unsigned long long c[4] = {0, 0, 0, 0};
-    HIP_CHECK(hipMemcpy(c, g_ws.counters, sizeof c, hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(c, g_ws.counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    c[1] = (jl.epilogue && c[0] > cap) ? cap : c[0];
+    c[2] = fasted::tile_count(n);
     float sortMs = 0.f;
     if ((flags & FASTED_SORT_PAIRS) && c[1] > 1) {
         const auto w0 = std::chrono::steady_clock::now();

@@ -17,7 +17,7 @@ struct JoinLaunch {
     int dPad;                    // K extent, multiple of kSlabK
     float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
     const float* sums;           // squared norms
-    unsigned long long* counters;  // counter_words() words: [0] found, [1] stored, [2] tiles done, queue heads
+    unsigned long long* counters;  // counter_words() words: [0] pairs found, then the queue heads
     void* pairs;                 // FastedPair[cap]
     unsigned long long cap;
     bool epilogue;               // false: contraction only (measurement)
@@ -27,6 +27,7 @@ struct JoinLaunch {
 unsigned long long raster_count(long long n);
 int raster_coord(unsigned long long idx, long long n, int* row, int* col);
 int counter_words();
+unsigned long long tile_count(long long n);  // 256x256 tiles the kernel processes
 // Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).
 int lds_chunk_slot(int row, int chunk);
 

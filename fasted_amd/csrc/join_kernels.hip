@@ -34,7 +34,11 @@ constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 
 constexpr int kLdsSums = 2 * kStageBytes;           // s_q[256] then s_c[256]
 constexpr int kLdsNext = kLdsSums + 2 * kTile * 4;  // next queue index
 constexpr int kLdsWaveMax = kLdsNext + 16;          // per-wave max of the tile's squared norms
-constexpr int kLdsBytes = kLdsWaveMax + 8 * 4;
+constexpr int kLdsStageCount = kLdsWaveMax + 8 * 4; // pairs waiting in the LDS staging area (u32) + flush base (u64)
+constexpr int kLdsStage = kLdsStageCount + 16;      // staged pairs
+constexpr int kStagePairs = 3072;                   // 24 KiB of 8-byte records
+constexpr int kLdsBytes = kLdsStage + kStagePairs * 8;
+static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
@@ -64,7 +68,7 @@ constexpr int kQueues = 8;                 // one per XCD
 constexpr int kSubRows = 4, kSubCols = 8;  // sub-rectangle of one XCD inside a super-square
 constexpr int kSubTiles = kSubRows * kSubCols;
 static_assert(kRaster == 16 && kSubTiles * kQueues == kRaster * kRaster, "8 sub-rectangles tile a super-square");
-constexpr int kCounterFound = 0, kCounterStored = 1, kCounterTiles = 2;
+constexpr int kCounterFound = 0;
 constexpr int kQueueBase = 16, kQueueStride = 16;  // queue heads sit on separate 128-byte lines
 constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
@@ -193,6 +197,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     float* const sC = sQ + kTile;
     unsigned long long* const sNext = reinterpret_cast<unsigned long long*>(lds + kLdsNext);
     float* const sWaveMax = reinterpret_cast<float*>(lds + kLdsWaveMax);
+    unsigned* const sStageCount = reinterpret_cast<unsigned*>(lds + kLdsStageCount);
+    unsigned long long* const sFlushBase = reinterpret_cast<unsigned long long*>(lds + kLdsStageCount + 8);
+    int2* const sStage = reinterpret_cast<int2*>(lds + kLdsStage);
 
     // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
     const unsigned home = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (kQueues - 1);
@@ -211,7 +218,25 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         return kDone;
     };
 
-    if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
+    // Pairs are staged in LDS and appended to the global list by the whole workgroup: one
+    // reservation on the global counter per flush instead of one per wave and tile, which is what
+    // bounds output-heavy joins (same-address atomics serialise at about 12 ns each).
+    auto flush_stage = [&](unsigned staged) {
+        const unsigned cnt = staged < (unsigned)kStagePairs ? staged : (unsigned)kStagePairs;
+        if (tid == 0) *sFlushBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)cnt);
+        __syncthreads();
+        const unsigned long long gb = *sFlushBase;
+        for (unsigned i = tid; i < cnt; i += kThreads)
+            if (gb + i < p.cap) p.pairs[gb + i] = sStage[i];  // past the capacity: counted, not stored
+        __syncthreads();
+        if (tid == 0) *sStageCount = 0u;
+        __syncthreads();
+    };
+
+    if (tid == 0) {
+        *sStageCount = 0u;
+        *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
+    }
     __syncthreads();
     unsigned long long ticket = *sNext;
 
@@ -392,19 +417,20 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                     const int v = __shfl_up(incl, off, 64);
                     if (lane >= off) incl += v;
                 }
-                const int total = __shfl(incl, 63, 64);
-                unsigned long long base = 0;
-                if (lane == 0) {
-                    base = atomicAdd(&p.counters[kCounterFound], (unsigned long long)total);
-                    // slots past the capacity are counted but not stored (source/pair.cuh:126-132)
-                    if (base < p.cap) {
-                        const unsigned long long room = p.cap - base;
-                        atomicAdd(&p.counters[kCounterStored],
-                                  room < (unsigned long long)total ? room : (unsigned long long)total);
-                    }
+                const unsigned total = (unsigned)__shfl(incl, 63, 64);
+                // reserve room in the staging area (LDS atomic); what does not fit goes straight
+                // to the global list with a reservation of this wave's own
+                unsigned pos = 0;
+                if (lane == 0) pos = atomicAdd(sStageCount, total);
+                pos = __shfl(pos, 0, 64);
+                const unsigned room = pos < (unsigned)kStagePairs ? (unsigned)kStagePairs - pos : 0u;
+                const unsigned fit = total < room ? total : room;
+                unsigned long long gbase = 0;
+                if (fit < total) {
+                    if (lane == 0) gbase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)(total - fit));
+                    gbase = __shfl(gbase, 0, 64);
                 }
-                base = __shfl(base, 0, 64);
-                unsigned long long slot = base + (unsigned long long)(incl - mine);
+                unsigned idx = (unsigned)(incl - mine);
 #pragma unroll
                 for (int fp = 0; fp < kFragRows / 2; ++fp) {
                     unsigned m = mask[fp];
@@ -414,8 +440,13 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         const int fi = fp * 2 + (bit >> 4), fj = (bit >> 2) & 3, r = bit & 3;
                         const int q = qBase + fi * 16 + quad * 4 + r;
                         const int c = colBase + wc * kWaveCols + fj * 16 + l16;
-                        if (slot < p.cap) p.pairs[slot] = make_int2(q, c);
-                        ++slot;
+                        if (idx < fit) {
+                            sStage[pos + idx] = make_int2(q, c);
+                        } else {
+                            const unsigned long long slot = gbase + (idx - fit);
+                            if (slot < p.cap) p.pairs[slot] = make_int2(q, c);
+                        }
+                        ++idx;
                     }
                 }
             }
@@ -426,10 +457,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) asm volatile("" ::"v"(acc[fi][fj]));
         }
-        if (tid == 0) atomicAdd(&p.counters[kCounterTiles], 1ull);
-
         __syncthreads();
         ticket = *sNext;
+        if (kEpilogue) {
+            const unsigned staged = *sStageCount;  // uniform: read after the barrier
+            if (staged >= (unsigned)kStagePairs / 2) flush_stage(staged);
+        }
+    }
+    if (kEpilogue) {
+        const unsigned staged = *sStageCount;
+        if (staged > 0) flush_stage(staged);
     }
 }
 
@@ -451,6 +488,11 @@ int raster_coord(unsigned long long idx, long long n, int* row, int* col) {
 }
 
 int counter_words() { return kCounterWords; }
+
+unsigned long long tile_count(long long n) {
+    const Raster r = make_raster(n);
+    return (unsigned long long)r.tilesPerDim * r.tilesPerDim;
+}
 
 int lds_chunk_slot(int row, int chunk) { return (chunk ^ swz(row)) & 7; }
 
