@@ -303,9 +303,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // One slab = 2 k-steps of 32; a k-step is two halves of 16 MFMAs (query blocks 0-3, then
         // 4-7, each against the 4 candidate blocks).  The instruction order is pinned with
         // scheduling barriers: the LDS reads for the next half are issued ahead of the MFMAs of
-        // the current half, and the 8 global->LDS transfers of the next slab are spread one per
-        // 8 MFMAs, so neither the LDS nor the texture-address queue makes a wave wait with the
-        // matrix pipe idle.
+        // the current half, and the 8 global->LDS transfers of the next slab are issued one per
+        // 4 MFMAs during the first k-step: spaced so that the texture-address queue never makes a
+        // wave wait with the matrix pipe idle, early so that an L2 miss has the whole second
+        // k-step to land before the slab's barrier.
         auto slab_step = [&](int s, auto prefetch) {
             constexpr bool kPrefetch = decltype(prefetch)::value;
             const unsigned nextByte = (unsigned)(s + 1) * kRowBytes;
@@ -325,7 +326,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) {
-                    if (kPrefetch && (fj & 1) == 0) issue_load(nextByte, (s + 1) & 1, ks * 4 + (fj >> 1));
+                    if (kPrefetch && ks == 0) issue_load(nextByte, (s + 1) & 1, fj);
 #pragma unroll
                     for (int fi = 0; fi < 4; ++fi)
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
@@ -342,7 +343,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) {
-                    if (kPrefetch && (fj & 1) == 0) issue_load(nextByte, (s + 1) & 1, ks * 4 + 2 + (fj >> 1));
+                    if (kPrefetch && ks == 0) issue_load(nextByte, (s + 1) & 1, 4 + fj);
 #pragma unroll
                     for (int fi = 0; fi < 4; ++fi)
                         acc[fi + 4][fj] =
