@@ -125,13 +125,15 @@ def cpu_baseline(torch, pts, eps, budget_s=15.0):
 
 
 def load_traffic(name):
-    """HBM bytes per join-kernel launch measured with rocprofv3 --pmc (committed under profiles/)."""
+    """Bytes below the L2 per join-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    and scaled by a plain copy kernel (committed under profiles/); None when not measured."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(name)
+            entry = json.load(f).get(name)
     except OSError:
-        return None
+        return None, None
+    return (entry["total"], entry) if entry else (None, None)
 
 
 def main():
@@ -178,7 +180,7 @@ def main():
     if args.n or args.d:
         label = f"{kind} {n}x{d} (override of {args.config})"
     pts = generate_points(torch, kind, n, d, seed=20260 + n % 997)
-    eps = args.eps or calibrate_epsilon(torch, pts, neighbours)
+    eps = args.eps or calibrate_epsilon(torch, pts, neighbours, sample=16384 if n >= 500_000 else 4096)
     # pair buffer: the reference's N*256 records, or 1.25x the expected count when that is larger
     cap = int(max(n * 256, 1.25 * n * (neighbours + 1)))
     pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
@@ -204,6 +206,7 @@ def main():
     join_ms = sum(s.joinMs for s in stats) / len(stats)
     sums_ms = sum(s.sumSquaredMs for s in stats) / len(stats)
     achieved = flops / (join_ms / 1000.0) / 1e12
+    traffic, traffic_detail = load_traffic(args.config if not (args.n or args.d) else "")
     out = {
         "metric": "self-join TFLOPS (2*N^2*D/s)", "value": tflops, "unit": "TFLOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -217,7 +220,7 @@ def main():
                    "accumulate": "f32", "peak_used_tflops": PEAK_FP16_TFLOPS},
         "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
-                     "traffic": load_traffic(args.config if not (args.n or args.d) else "")},
+                     "traffic": traffic, "traffic_detail": traffic_detail},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
