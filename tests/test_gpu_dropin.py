@@ -1,0 +1,87 @@
+"""GPU tests of the drop-in boundary: the reference's entry points, the `.pairs` text output and the
+command-line driver, checked against the CPU checker."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle
+from tests import datasets
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import fasted_amd
+
+    return fasted_amd.load_findpairs()
+
+
+def write_csv(path, values):
+    with open(path, "w") as f:
+        for row in values:
+            f.write(",".join(repr(float(v)) for v in row) + "\n")
+
+
+def test_run_from_file_saves_sorted_pairs_text(lib, tmp_path):
+    import fasted_amd
+
+    rng = np.random.default_rng(21)
+    vals = np.round(rng.random((900, 40)), 6)
+    csv = tmp_path / "points900.csv"
+    write_csv(csv, vals)
+    bits = oracle.quantize(vals)
+    eps = datasets.epsilon_for_neighbours(bits, 6)
+    lib.fasted_set_output_dir(str(tmp_path).encode())
+    r = lib.runFromFile(str(csv).encode(), eps, True)
+    assert (r.inputProblemShape.m, r.inputProblemShape.k) == (900, 40)
+    assert (r.paddedProblemShape.m, r.paddedProblemShape.k) == (1024, 64)
+    assert r.pairsFound == r.pairsStored
+    # file name: <dataset name>_<std::to_string(eps)>.pairs ; lines "q, c"
+    out = tmp_path / ("points900_%f.pairs" % eps)
+    assert out.exists(), os.listdir(tmp_path)
+    text = out.read_text().splitlines()
+    assert all(re.fullmatch(r"\d+, \d+", line) for line in text)
+    got = np.array([[int(x) for x in line.split(", ")] for line in text], dtype=np.int32)
+    assert len(got) == r.pairsFound
+    assert np.array_equal(got, oracle.sort_pairs(got))  # already row-major
+    rep = oracle.epsilon_band_report(bits, got, eps)
+    assert rep["outside_band"] == 0 and rep["both"] > 900
+    # the resident dataset is what the reference's builder would hold
+    resident, n, d, name = fasted_amd.resident_points()
+    assert (n, d, name) == (900, 40, "points900")
+    assert np.array_equal(resident[:900, :40], bits)
+    # reRun on the resident data, no file this time
+    r2 = lib.reRun(eps * 1.1, False)
+    assert r2.pairsFound > r.pairsFound
+    assert len(list(tmp_path.glob("*.pairs"))) == 1
+    lib.releaseResources()
+    lib.fasted_set_output_dir(b"")
+
+
+def test_results_fields_and_tflops_formula(lib):
+    n, d = 5000, 256
+    r = lib.runFromExponentialDataset(n, d, 40.0, 10.0, 0.5, False)
+    assert r.totalTime > 0
+    # TFLOPS = 2 N^2 D / kernel time with unpadded N, D: kernel time must be below the total time
+    kernel_s = 2.0 * n * n * d / (r.TFLOPS * 1e12)
+    assert 0 < kernel_s <= r.totalTime
+    assert r.get_selectivity() == max(0, r.pairsFound - n) / n
+    lib.releaseResources()
+
+
+def test_command_line_driver(tmp_path):
+    exe = os.path.join(ROOT, "fasted_amd", "fasted")
+    assert os.path.exists(exe), "build the CLI with make -C fasted_amd/csrc release"
+    out = subprocess.run([exe, "-e", "3000", "128", "0.001"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "Pairs found: 3000" in out.stdout  # only the self pairs at eps = 0.001
+    assert re.search(r"Estimated TFLOPS [\d.]+", out.stdout)
+    bad = subprocess.run([exe, "-e", "10"], capture_output=True, text=True, timeout=60)
+    assert bad.returncode == 1 and "Usage" in bad.stderr
+    missing = subprocess.run([exe, str(tmp_path / "nope.csv"), "0.1"], capture_output=True, text=True, timeout=60)
+    assert missing.returncode != 0 and "Failed" in missing.stdout
