@@ -11,6 +11,8 @@ from .find_pairs import (  # noqa: F401
     RerunnablePairsFinder,
     Results,
     compute_selectivity,
+    count_pairs,
+    find_epsilon,
     library_path,
     load_findpairs,
     mmaShape,
@@ -21,6 +23,6 @@ from .find_pairs import (  # noqa: F401
 )
 
 __all__ = [
-    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "library_path",
+    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "library_path",
     "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_device", "sum_squared_device",
 ]

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <cmath>
 #include <climits>
 #include <cstdio>
 #include <cstdlib>
@@ -290,6 +291,34 @@ Results run_source(fasted::PointSource* src, double epsilon, bool savePairs) {
     }
 }
 
+// Uploads the resident dataset if it is not on the device yet.
+void ensure_resident_uploaded() {
+    const fasted::PointTable& tb = g_res.table;
+    if (tb.empty()) throw std::runtime_error("no dataset is resident: call runFromFile or runFromExponentialDataset first");
+    if (g_res.uploaded) return;
+    HIP_CHECK(hipSetDevice(0));
+    g_res.drop_device();
+    const size_t bytes = tb.bits.size() * sizeof(uint16_t);
+    HIP_CHECK(hipMalloc(&g_res.dPoints, bytes));
+    HIP_CHECK(hipMemcpy(g_res.dPoints, tb.bits.data(), bytes, hipMemcpyHostToDevice));
+    g_res.uploaded = true;
+}
+
+// One join on the resident dataset that only counts: no pair buffer, no sort, no download.
+FastedJoinStats count_resident(double epsilon) {
+    ensure_resident_uploaded();
+    const fasted::PointTable& tb = g_res.table;
+    FastedJoinStats st{};
+    join_on_device(g_res.dPoints, tb.n, tb.dPad, tb.dPad, epsilon, nullptr, nullptr, 0, 0, nullptr, &st);
+    return st;
+}
+
+double selectivity_of(unsigned long long pairsFound, int n) {
+    // (|R| - |D|) / |D|, never negative (results/scripts/experiment/find_pairs.py:9-21)
+    const double r = (double)pairsFound - (double)n;
+    return (r > 0 ? r : 0.0) / (double)n;
+}
+
 template <typename F>
 int guarded(F&& body) {
     try {
@@ -404,6 +433,55 @@ int fasted_load_file(const char* filename) {
 }
 
 const char* fasted_resident_name(void) { return g_res.table.name.c_str(); }
+
+int fasted_count_pairs(double epsilon, unsigned long long* pairsFound, double* kernelSeconds) {
+    return guarded([&] {
+        const FastedJoinStats st = count_resident(epsilon);
+        if (pairsFound) *pairsFound = st.pairsFound;
+        if (kernelSeconds) *kernelSeconds = (st.sumSquaredMs + st.joinMs) / 1000.0;
+    });
+}
+
+int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
+                        int* probes) {
+    return guarded([&] {
+        if (!(targetSelectivity > 0.0)) throw std::invalid_argument("target selectivity must be positive");
+        if (initialEpsilon < 0.0) throw std::invalid_argument("initial epsilon must not be negative");
+        const int n = g_res.table.n;
+        int count = 0;
+        auto probe = [&](double eps) {
+            ++count;
+            return selectivity_of(count_resident(eps).pairsFound, n);
+        };
+        // bound: double epsilon (0 -> 2) until the target is reached (experiments.py:153-195)
+        const double maxEpsilon = 100000.0;
+        double lower = initialEpsilon, upper = initialEpsilon, current = 0.0;
+        while (current < targetSelectivity) {
+            lower = upper;
+            upper = (lower == 0.0) ? 2.0 : lower * 2.0;
+            if (upper > maxEpsilon)
+                throw std::runtime_error("Epsilon of " + std::to_string(upper) + " exceed the maximum value of " +
+                                         std::to_string(maxEpsilon) + ". Giving up trying to find the upper bound.");
+            current = probe(upper);
+        }
+        // bisect by half steps until within 1 % of the target (experiments.py:198-281)
+        double eps = (upper - lower) / 2.0 + lower, last = upper;
+        current = probe(eps);
+        int guard = 0;
+        while (!(std::fabs(current - targetSelectivity) / targetSelectivity < 0.01)) {
+            const double step = std::fabs(eps - last);
+            const double next = current > targetSelectivity ? eps - 0.5 * step : eps + 0.5 * step;
+            last = eps;
+            eps = next;
+            if (++guard > 200 || next == last)  // the reference would loop forever on a plateau
+                throw std::runtime_error("epsilon search did not converge to within 1% of the target selectivity");
+            current = probe(eps);
+        }
+        if (epsilon) *epsilon = eps;
+        if (selectivity) *selectivity = current;
+        if (probes) *probes = count;
+    });
+}
 
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     if (n < 1 || !row || !col) return 0;

@@ -122,6 +122,11 @@ def load_findpairs(path: str = None):
     lib.fasted_load_exponential_dataset.argtypes = [c.c_int, c.c_int, c.c_double, c.c_double]
     lib.fasted_load_file.restype = c.c_int
     lib.fasted_load_file.argtypes = [c.c_char_p]
+    lib.fasted_count_pairs.restype = c.c_int
+    lib.fasted_count_pairs.argtypes = [c.c_double, c.POINTER(c.c_ulonglong), c.POINTER(c.c_double)]
+    lib.fasted_find_epsilon.restype = c.c_int
+    lib.fasted_find_epsilon.argtypes = [c.c_double, c.c_double, c.POINTER(c.c_double), c.POINTER(c.c_double),
+                                        c.POINTER(c.c_int)]
     lib.fasted_resident_name.restype = c.c_char_p
     lib.fasted_resident_points.restype = c.c_void_p
     lib.fasted_resident_points.argtypes = [c.POINTER(c.c_int)] * 4
@@ -183,6 +188,23 @@ def resident_points():
         return None
     arr = np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_uint16)), (n_pad.value, d_pad.value))
     return arr.copy(), n.value, d.value, lib.fasted_resident_name().decode()
+
+
+def count_pairs(epsilon):
+    """Count-only join on the resident dataset: (pairsFound, kernel seconds)."""
+    lib = load_findpairs()
+    found, secs = ctypes.c_ulonglong(), ctypes.c_double()
+    _check(lib, lib.fasted_count_pairs(float(epsilon), ctypes.byref(found), ctypes.byref(secs)))
+    return found.value, secs.value
+
+
+def find_epsilon(target_selectivity, initial_epsilon=0.0):
+    """Native bound-then-bisect epsilon search on the resident dataset: (epsilon, selectivity, probes)."""
+    lib = load_findpairs()
+    eps, sel, probes = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
+    _check(lib, lib.fasted_find_epsilon(float(target_selectivity), float(initial_epsilon), ctypes.byref(eps),
+                                        ctypes.byref(sel), ctypes.byref(probes)))
+    return eps.value, sel.value, probes.value
 
 
 def sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream=None):

@@ -135,6 +135,20 @@ int fasted_lds_chunk_slot(int row, int chunk);
 int fasted_load_exponential_dataset(int size, int dimensionality, double lambda, double max);
 int fasted_load_file(const char* filename);
 
+/* Count-only join on the resident dataset (no pair buffer, no sort, no download): *pairsFound as
+ * reRun() would report it, *kernelSeconds = squared norms + join kernel.  The probe an epsilon
+ * search needs; the reference pays a full reRun for it (results/scripts/experiment/
+ * experiments.py:153-281 call find_pairs once per probe). */
+int fasted_count_pairs(double epsilon, unsigned long long* pairsFound, double* kernelSeconds);
+
+/* Epsilon for a target selectivity (mean neighbours per point, self pairs excluded) on the resident
+ * dataset: the bound-then-bisect search of the reference's find_epsilon_binary
+ * (results/scripts/experiment/experiments.py:153-281: double from `initialEpsilon` (0 -> 2) until
+ * the target is reached, then half steps until within 1 %), with count-only probes.  Fails instead
+ * of looping forever when the selectivity cannot come within 1 % of the target. */
+int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
+                        int* probes);
+
 /* Resident dataset: padded FP16 bit patterns (host copy) and its name
  * (PointGenerator::getName, source/DataLoader/PointGenerator.hpp:27-30). */
 const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad);

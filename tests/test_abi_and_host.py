@@ -202,3 +202,54 @@ def test_lds_swizzle_is_a_bijection_and_bank_conflict_free(lib):
                 touched = {((base + l % 16) & 1, lib.fasted_lds_chunk_slot(base + l % 16, 4 * ks + l // 16))
                            for l in phase}
                 assert len(touched) == 16, (base, ks, phase)
+
+
+# ---------------------------------------------------------------- epsilon search + accuracy helpers
+class MockFindPairs:
+    """Stand-in backend in the manner of the reference's tests (results/scripts/tests/
+    test_experiments.py:14-71): pairsFound is a monotone function of epsilon."""
+
+    def __init__(self, n=10_000, density=700.0):
+        self.n, self.density, self.calls = n, density, []
+
+    def selectivity(self, eps):
+        self.calls.append(eps)
+        found = int(self.n + self.density * eps ** 3 * self.n)
+        return fp.compute_selectivity(found, self.n)
+
+
+def test_epsilon_search_follows_the_reference_procedure():
+    from fasted_amd import experiments as ex
+
+    assert ex.within_percent(100.5, 100, 0.01) and not ex.within_percent(102, 100, 0.01)
+    assert ex.adjust_epsilon_binary(4.0, 8.0, 64, 100) == 2.0  # overshoot: half a step back
+    assert ex.adjust_epsilon_binary(2.0, 4.0, 64, 10) == 3.0   # undershoot: half a step forward
+    mock = MockFindPairs()
+    lo, hi = ex.bound_epsilon(0.0, 100000, 64, mock.selectivity)
+    assert mock.calls == [2.0] and (lo, hi) == (0.0, 2.0)  # 0 -> 2, then doubling
+    mock = MockFindPairs(density=0.001)
+    assert ex.bound_epsilon(0.0, 100000, 64, mock.selectivity) == (32.0, 64.0)
+    assert mock.calls == [2.0, 4.0, 8.0, 16.0, 32.0, 64.0]
+    with pytest.raises(ValueError):
+        ex.bound_epsilon(0.0, 10.0, 1e12, MockFindPairs().selectivity)
+    mock = MockFindPairs()
+    eps = ex.find_epsilon_binary(64, mock.selectivity)
+    assert ex.within_percent(700.0 * eps ** 3, 64, 0.011)
+    assert mock.calls[:2] == [2.0, 1.0]  # the upper bound, then the midpoint of (0, 2)
+
+
+def test_pair_statistics_and_per_point_iou():
+    from fasted_amd import experiments as ex
+
+    five = np.array([[1, 1], [2, 2], [3, 3], [4, 4], [5, 5]])
+    assert ex.compute_pair_stats(five, five) == ex.PairsStats(5, 0, 0, 5, 5)
+    assert ex.compute_pair_stats(five, np.delete(five, 2, axis=0)) == ex.PairsStats(4, 0, 1, 5, 4)
+    assert ex.compute_pair_stats(np.delete(five, 0, axis=0), five) == ex.PairsStats(4, 1, 0, 4, 5)
+    # agrees with the checker's merge walk on random lists
+    rng = np.random.default_rng(9)
+    a = oracle.sort_pairs(np.unique(rng.integers(0, 40, (300, 2)), axis=0))
+    b = oracle.sort_pairs(np.unique(rng.integers(0, 40, (300, 2)), axis=0))
+    s, o = ex.compute_pair_stats(a, b), oracle.pair_stats(a, b)
+    assert (s.both_sides, s.right_only, s.left_only) == (o["both"], o["right_only"], o["left_only"])
+    iou = ex.per_point_iou([[0, 0], [0, 1], [1, 1], [2, 2]], [[0, 0], [0, 2], [1, 1]], 4)
+    assert iou.tolist() == [1 / 3, 1.0, 0.0, 1.0]

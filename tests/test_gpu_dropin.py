@@ -85,3 +85,31 @@ def test_command_line_driver(tmp_path):
     assert bad.returncode == 1 and "Usage" in bad.stderr
     missing = subprocess.run([exe, str(tmp_path / "nope.csv"), "0.1"], capture_output=True, text=True, timeout=60)
     assert missing.returncode != 0 and "Failed" in missing.stdout
+
+
+def test_native_epsilon_search_matches_the_python_procedure(lib):
+    """fasted_find_epsilon follows the reference's bound-then-bisect search probe for probe: the
+    Python mirror driven by count-only probes lands on the same epsilon."""
+    import fasted_amd
+    from fasted_amd import experiments as ex
+
+    n, d = 6000, 64
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    eps, sel, probes = fasted_amd.find_epsilon(16.0)
+    assert ex.within_percent(sel, 16.0, 0.01) and probes >= 3
+    calls = []
+
+    def get_selectivity(e):
+        calls.append(e)
+        return fasted_amd.compute_selectivity(fasted_amd.count_pairs(e)[0], n)
+
+    assert ex.find_epsilon_binary(16.0, get_selectivity) == eps
+    assert len(calls) == probes
+    # the count-only probe agrees with a storing reRun and with the FP64 checker
+    found, secs = fasted_amd.count_pairs(eps)
+    r = lib.reRun(eps, False)
+    assert found == r.pairsFound and secs > 0
+    bits, _, _, _ = fasted_amd.resident_points()
+    truth = oracle.self_join_f64(bits, eps, n=n)
+    assert abs(int(found) - len(truth)) <= max(4, len(truth) // 500)
+    lib.releaseResources()
