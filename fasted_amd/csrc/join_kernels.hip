@@ -135,13 +135,26 @@ struct JoinParams {
 };
 
 // Distance test of one wave's 128x64 block of accumulators.  acc[fi][fj] is a 16x16 MFMA block:
-// lane l holds column l%16 and rows 4*(l/16) .. +3.  kEdge: the tile touches the diagonal or the
-// ragged end of the dataset, so self pairs are forced and padded rows/cols are masked
-// (source/warpMma.cuh:257-259).  Returns per-lane hit bits: mask[fi/2] bit ((fi&1)*16 + fj*4 + r).
+// lane l holds column l%16 and rows 4*(l/16) .. +3, i.e. 4 elements per block.
+//
+// Screening, 1.75 VALU ops per element: in real arithmetic a hit is
+//     acc - s_q/2 >= (s_c - eps^2)/2,
+// so per block the maximum of acc - s_q/2 over the lane's 4 rows is compared with the column's
+// right-hand side minus `margin`, which covers every FP32 rounding of both forms.  The compare is
+// wave-wide (its result is the ballot), and only blocks in which some lane has a candidate evaluate
+// the reference formula exactly:  (s_q + s_c) - 2*acc <= eps^2  in FP32 (source/warpMma.cuh:241-257).
+//
+// kEdge: the tile touches the diagonal or the ragged end of the dataset; every block is evaluated
+// exactly, self pairs are forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
+// Returns per-lane hit bits: mask[fi/2] bit ((fi&1)*16 + fj*4 + r).
 template <bool kEdge>
 __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const float* sQ,
                                            const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
-                                           int quad, int n, float eps2, unsigned (&mask)[kFragRows / 2]) {
+                                           int quad, int n, float eps2, float margin,
+                                           unsigned (&mask)[kFragRows / 2]) {
+    float thr[kFragCols];
+#pragma unroll
+    for (int fj = 0; fj < kFragCols; ++fj) thr[fj] = 0.5f * (sc[fj] - eps2) - margin;
 #pragma unroll
     for (int fp = 0; fp < kFragRows / 2; ++fp) {
         unsigned m = 0;
@@ -149,18 +162,26 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
         for (int h = 0; h < 2; ++h) {
             const int fi = fp * 2 + h;
             const floatx4 sq = *reinterpret_cast<const floatx4*>(sQ + fi * 16 + quad * 4);
+            const floatx4 hq = sq * 0.5f;
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj) {
+                bool look = kEdge;
+                if (!kEdge) {
+                    const floatx4 f = acc[fi][fj] - hq;
+                    const float best = __builtin_fmaxf(__builtin_fmaxf(f[0], f[1]), __builtin_fmaxf(f[2], f[3]));
+                    look = __builtin_amdgcn_ballot_w64(best >= thr[fj]) != 0ull;
+                }
+                if (look) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    // (s_q + s_c) - 2*acc, FP32, as source/warpMma.cuh:241-242
-                    const float d2 = (sq[r] + sc[fj]) - (2.0f * acc[fi][fj][r]);
-                    bool hit = d2 <= eps2;
-                    if (kEdge) {
-                        const int q = qBase + fi * 16 + quad * 4 + r;
-                        hit = (hit || q == cand[fj]) && q < n && cand[fj] < n;
+                    for (int r = 0; r < 4; ++r) {
+                        const float d2 = (sq[r] + sc[fj]) - (2.0f * acc[fi][fj][r]);
+                        bool hit = d2 <= eps2;
+                        if (kEdge) {
+                            const int q = qBase + fi * 16 + quad * 4 + r;
+                            hit = (hit || q == cand[fj]) && q < n && cand[fj] < n;
+                        }
+                        m = hit ? (m | (1u << (h * 16 + fj * 4 + r))) : m;
                     }
-                    m = hit ? (m | (1u << (h * 16 + fj * 4 + r))) : m;
                 }
             }
         }
@@ -366,46 +387,17 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
                 sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
             }
-            // Screening pass (1.5 VALU ops per element): in real arithmetic a hit is
-            //   acc - s_q/2 >= (s_c - eps^2)/2,
-            // so take the per-column maximum of acc - s_q/2 and compare it, with a margin that
-            // covers every FP32 rounding of both forms, against the column's right-hand side.
-            // Only waves with a candidate run the exact reference formula below; on tiles that
-            // touch the diagonal or the ragged end every wave does.
+            // margin of the screening test: covers the FP32 roundings of both forms of the inequality
             const bool edge = (tr == tc) || rowBase + kTile > p.n || colBase + kTile > p.n;
-            bool candidate = edge;
-            if (!edge) {
-                float sMax = sWaveMax[0];
+            float sMax = sWaveMax[0];
 #pragma unroll
-                for (int w = 1; w < 8; ++w) sMax = __builtin_fmaxf(sMax, sWaveMax[w]);
-                const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
-                float best[kFragCols];
-#pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) best[fj] = -__builtin_inff();
-#pragma unroll
-                for (int fi = 0; fi < kFragRows; ++fi) {
-                    const floatx4 hq = *reinterpret_cast<const floatx4*>(sQ + wr * kWaveRows + fi * 16 + quad * 4) * 0.5f;
-#pragma unroll
-                    for (int fj = 0; fj < kFragCols; ++fj) {
-                        const floatx4 f = acc[fi][fj] - hq;
-                        best[fj] = __builtin_fmaxf(best[fj], __builtin_fmaxf(__builtin_fmaxf(f[0], f[1]),
-                                                                             __builtin_fmaxf(f[2], f[3])));
-                    }
-                }
-                bool any = false;
-#pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) any = any || (best[fj] >= 0.5f * (sc[fj] - p.eps2) - margin);
-                candidate = __builtin_amdgcn_ballot_w64(any) != 0ull;
-            }
+            for (int w = 1; w < 8; ++w) sMax = __builtin_fmaxf(sMax, sWaveMax[w]);
+            const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
             unsigned mask[kFragRows / 2];
-#pragma unroll
-            for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
-            if (candidate) {
-                if (edge)
-                    test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
-                else
-                    test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, mask);
-            }
+            if (edge)
+                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, margin, mask);
+            else
+                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, margin, mask);
 
             int mine = 0;
 #pragma unroll
