@@ -92,6 +92,39 @@ def calibrate_epsilon(torch, pts, neighbours, sample=4096, seed=4242):
     return math.sqrt(eps2)
 
 
+def parity_sample(torch, pts, eps, pairs, stored, rows=256, seed=7, band=1e-3):
+    """Pair-set check of `rows` seeded query rows against FP64 distances to all points (torch FP64 on
+    the device, outside the timed region): pairs that disagree with FP64, how many of them lie outside
+    the relative `band` around epsilon (must be 0), and the largest relative distance error."""
+    n, d = pts.shape
+    got = pairs[:stored]
+    order = torch.argsort(got[:, 0].to(torch.int64) * n + got[:, 1].to(torch.int64))
+    q = got[order, 0].to(torch.int64).contiguous()
+    c = got[order, 1].to(torch.int64)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    sel = torch.sort(torch.randperm(n, generator=g, device="cuda")[:rows]).values
+    start, stop = torch.searchsorted(q, sel), torch.searchsorted(q, sel + 1)
+    mask = torch.zeros((len(sel), n), dtype=torch.bool, device="cuda")
+    for i in range(len(sel)):
+        mask[i, c[start[i]:stop[i]]] = True
+    xs = pts[sel].to(torch.float64)
+    xs2 = (xs * xs).sum(1)
+    disagree, outside, worst = 0, 0, 0.0
+    chunk = max(1, (1 << 26) // d)
+    for c0 in range(0, n, chunk):
+        y = pts[c0:c0 + chunk].to(torch.float64)
+        d2 = (xs2[:, None] + (y * y).sum(1)[None, :] - 2.0 * (xs @ y.T)).clamp_min(0.0)
+        diff = (d2 <= eps * eps) != mask[:, c0:c0 + chunk]
+        if bool(diff.any()):
+            rel = (d2[diff].sqrt() - eps).abs() / eps
+            disagree += int(diff.sum())
+            outside += int((rel > band).sum())
+            worst = max(worst, float(rel.max()))
+    return {"rows": int(len(sel)), "pairs_checked": int((stop - start).sum()), "disagree_with_fp64": disagree,
+            "outside_band": outside, "max_rel_distance_error": worst, "band": band}
+
+
 def cpu_baseline(torch, pts, eps, budget_s=15.0):
     """FP64 brute-force join (the CPU checker) on a bounded sample: Q query rows against the
     first Nc points of the same dataset, on this box's host cores."""
@@ -222,6 +255,8 @@ def main():
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": traffic, "traffic_detail": traffic_detail},
     }
+    if not args.no_epilogue and st.pairsStored == st.pairsFound:
+        out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
     print(json.dumps(out))
