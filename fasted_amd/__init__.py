@@ -13,6 +13,7 @@ from .find_pairs import (  # noqa: F401
     compute_selectivity,
     count_pairs,
     find_epsilon,
+    join_device,
     library_path,
     load_findpairs,
     mmaShape,
@@ -23,6 +24,6 @@ from .find_pairs import (  # noqa: F401
 )
 
 __all__ = [
-    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "library_path",
+    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "join_device", "library_path",
     "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_device", "sum_squared_device",
 ]

@@ -103,30 +103,49 @@ void validate_shape(long long n, int d, long long ld) {
     if ((ld / 8) * fasted::kTile >= (1ll << 31)) throw std::invalid_argument("row stride too large");
 }
 
+// One side of a join: `n` FP16 rows of `d` dimensions, row stride `ld` halves.
+struct PointSet {
+    const void* ptr;
+    long long n;
+    long long ld;
+    float* sums;  // caller's buffer for the squared norms, or null
+};
+
 // The timed region of the reference (source/findPairs.cuh:625-697): squared norms, then
 // queue/pair-counter reset and the join kernel; then counters come back and the stored pairs
-// are sorted outside the TFLOPS window.
-void join_on_device(const void* dPoints, long long n, int d, long long ld, double epsilon, float* dSums, void* dPairs,
+// are sorted outside the TFLOPS window.  `c.ptr == q.ptr` with selfJoin computes the norms once.
+void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon, void* dPairs,
                     unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats) {
-    validate_shape(n, d, ld);
+    validate_shape(q.n, d, q.ld);
+    validate_shape(c.n, d, c.ld);
     if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
     const int dPad = round_up(d, fasted::kSlabK);
-    g_ws.ensure((size_t)n);
-    float* sums = dSums ? dSums : g_ws.sums;
-    if ((flags & FASTED_SKIP_SUMS) && !dSums) throw std::invalid_argument("FASTED_SKIP_SUMS needs d_sums");
+    g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
+    float* sumsQ = q.sums ? q.sums : g_ws.sums;
+    float* sumsC = selfJoin ? sumsQ : (c.sums ? c.sums : g_ws.sums + q.n);
+    if ((flags & FASTED_SKIP_SUMS) && (!q.sums || (!selfJoin && !c.sums)))
+        throw std::invalid_argument("FASTED_SKIP_SUMS needs the squared-norm buffers");
 
     EventTimer t;
     HIP_CHECK(hipEventRecord(t.ev[0], stream));
-    if (!(flags & FASTED_SKIP_SUMS)) HIP_CHECK(fasted::launch_sum_squared(dPoints, ld, (int)n, dPad, sums, stream));
+    if (!(flags & FASTED_SKIP_SUMS)) {
+        HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, stream));
+        if (!selfJoin) HIP_CHECK(fasted::launch_sum_squared(c.ptr, c.ld, (int)c.n, dPad, sumsC, stream));
+    }
     HIP_CHECK(hipEventRecord(t.ev[1], stream));
 
     fasted::JoinLaunch jl;
-    jl.points = dPoints;
-    jl.ld = ld;
-    jl.n = (int)n;
+    jl.queries = q.ptr;
+    jl.candidates = c.ptr;
+    jl.ldQ = q.ld;
+    jl.ldC = c.ld;
+    jl.nQ = (int)q.n;
+    jl.nC = (int)c.n;
+    jl.selfJoin = selfJoin;
     jl.dPad = dPad;
     jl.eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
-    jl.sums = sums;
+    jl.sumsQ = sumsQ;
+    jl.sumsC = sumsC;
     jl.counters = g_ws.counters;
     jl.pairs = dPairs;
     jl.cap = cap;
@@ -138,25 +157,25 @@ void join_on_device(const void* dPoints, long long n, int d, long long ld, doubl
 
     // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
     // counted only (source/pair.cuh:123-133), so stored = min(found, capacity)
-    unsigned long long c[4] = {0, 0, 0, 0};
-    HIP_CHECK(hipMemcpy(c, g_ws.counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
-    c[1] = (jl.epilogue && c[0] > cap) ? cap : c[0];
-    c[2] = fasted::tile_count(n);
+    unsigned long long cnt[4] = {0, 0, 0, 0};
+    HIP_CHECK(hipMemcpy(cnt, g_ws.counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
+    cnt[2] = fasted::tile_count(q.n, c.n);
     float sortMs = 0.f;
-    if ((flags & FASTED_SORT_PAIRS) && c[1] > 1) {
+    if ((flags & FASTED_SORT_PAIRS) && cnt[1] > 1) {
         const auto w0 = std::chrono::steady_clock::now();
-        HIP_CHECK(fasted::sort_pairs_row_major(dPairs, c[1], stream));
+        HIP_CHECK(fasted::sort_pairs_row_major(dPairs, cnt[1], stream));
         sortMs = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
     }
     if (stats) {
         stats->sumSquaredMs = t.ms(0, 1);
         stats->joinMs = t.ms(1, 2);
         stats->sortMs = sortMs;
-        stats->paddedN = round_up(n, fasted::kTile);
+        stats->paddedN = round_up(q.n, fasted::kTile);
         stats->paddedD = dPad;
-        stats->tiles = c[2];
-        stats->pairsFound = c[0];
-        stats->pairsStored = c[1];
+        stats->tiles = cnt[2];
+        stats->pairsFound = cnt[0];
+        stats->pairsStored = cnt[1];
     }
 }
 
@@ -219,8 +238,8 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
     FastedJoinStats st{};
     std::vector<FastedPair> pairs;
     try {
-        join_on_device(g_res.dPoints, tb.n, tb.dPad, tb.dPad, epsilon, nullptr, dPairs, maxPairs, FASTED_SORT_PAIRS,
-                       nullptr, &st);
+        const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
+        join_on_device(all, all, true, tb.dPad, epsilon, dPairs, maxPairs, FASTED_SORT_PAIRS, nullptr, &st);
         if (!quiet()) {
             std::printf("Number of pairs found %llu\n", st.pairsFound);
             std::printf("Number of pairs stored %llu\n", st.pairsStored);
@@ -309,7 +328,8 @@ FastedJoinStats count_resident(double epsilon) {
     ensure_resident_uploaded();
     const fasted::PointTable& tb = g_res.table;
     FastedJoinStats st{};
-    join_on_device(g_res.dPoints, tb.n, tb.dPad, tb.dPad, epsilon, nullptr, nullptr, 0, 0, nullptr, &st);
+    const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
+    join_on_device(all, all, true, tb.dPad, epsilon, nullptr, 0, 0, nullptr, &st);
     return st;
 }
 
@@ -368,8 +388,20 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
                             FastedJoinStats* stats) {
     return guarded([&] {
         if (!d_points) throw std::invalid_argument("points pointer is null");
-        join_on_device(d_points, n, d, ld, epsilon, d_sums, d_pairs, cap, flags, static_cast<hipStream_t>(stream),
-                       stats);
+        const PointSet all{d_points, n, ld, d_sums};
+        join_on_device(all, all, true, d, epsilon, d_pairs, cap, flags, static_cast<hipStream_t>(stream), stats);
+    });
+}
+
+int fasted_join_device(const void* d_queries, long long n_queries, long long ld_queries, const void* d_candidates,
+                       long long n_candidates, long long ld_candidates, int d, double epsilon, float* d_sums_queries,
+                       float* d_sums_candidates, FastedPair* d_pairs, unsigned long long cap, unsigned flags,
+                       void* stream, FastedJoinStats* stats) {
+    return guarded([&] {
+        if (!d_queries || !d_candidates) throw std::invalid_argument("points pointer is null");
+        const PointSet q{d_queries, n_queries, ld_queries, d_sums_queries};
+        const PointSet c{d_candidates, n_candidates, ld_candidates, d_sums_candidates};
+        join_on_device(q, c, false, d, epsilon, d_pairs, cap, flags, static_cast<hipStream_t>(stream), stats);
     });
 }
 
@@ -401,7 +433,8 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
                                   hipMemcpyHostToDevice));
             HIP_CHECK(hipMalloc(&dPairs, (size_t)(cap ? cap : 1) * sizeof(FastedPair)));
             FastedJoinStats st{};
-            join_on_device(dPoints, n, d, dPad, epsilon, nullptr, dPairs, cap, FASTED_SORT_PAIRS, nullptr, &st);
+            const PointSet all{dPoints, n, dPad, nullptr};
+            join_on_device(all, all, true, d, epsilon, dPairs, cap, FASTED_SORT_PAIRS, nullptr, &st);
             if (st.pairsStored)
                 HIP_CHECK(hipMemcpy(out, dPairs, (size_t)st.pairsStored * sizeof(FastedPair), hipMemcpyDeviceToHost));
             if (found) *found = st.pairsFound;
@@ -485,12 +518,12 @@ int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double*
 
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     if (n < 1 || !row || !col) return 0;
-    return fasted::raster_coord(idx, n, row, col);
+    return fasted::raster_coord(idx, n, n, row, col);
 }
 
 int fasted_lds_chunk_slot(int row, int chunk) { return fasted::lds_chunk_slot(row, chunk); }
 
-unsigned long long fasted_raster_count(long long n) { return n < 1 ? 0ull : fasted::raster_count(n); }
+unsigned long long fasted_raster_count(long long n) { return n < 1 ? 0ull : fasted::raster_count(n, n); }
 
 const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad) {
     const fasted::PointTable& tb = g_res.table;

@@ -11,12 +11,15 @@ constexpr int kSlabK = 64;       // halves of K staged in LDS per pipeline stage
 constexpr int kRaster = 16;      // tiles per side of a raster square
 
 struct JoinLaunch {
-    const void* points;          // FP16 rows
-    long long ld;                // row stride in halves (multiple of 8)
-    int n;                       // real points
+    const void* queries;         // FP16 rows
+    const void* candidates;      // FP16 rows; the same buffer for a self-join
+    long long ldQ, ldC;          // row strides in halves (multiples of 8)
+    int nQ, nC;                  // real points
+    bool selfJoin;               // same set on both sides: (i, i) always counts as a pair
     int dPad;                    // K extent, multiple of kSlabK
     float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
-    const float* sums;           // squared norms
+    const float* sumsQ;          // squared norms of the queries
+    const float* sumsC;          // ... of the candidates
     unsigned long long* counters;  // counter_words() words: [0] pairs found, then the queue heads
     void* pairs;                 // FastedPair[cap]
     unsigned long long cap;
@@ -24,10 +27,10 @@ struct JoinLaunch {
 };
 
 // Host mirror of the device tile order.
-unsigned long long raster_count(long long n);
-int raster_coord(unsigned long long idx, long long n, int* row, int* col);
+unsigned long long raster_count(long long nQ, long long nC);
+int raster_coord(unsigned long long idx, long long nQ, long long nC, int* row, int* col);
 int counter_words();
-unsigned long long tile_count(long long n);  // 256x256 tiles the kernel processes
+unsigned long long tile_count(long long nQ, long long nC);  // 256x256 tiles the kernel processes
 // Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).
 int lds_chunk_slot(int row, int chunk);
 

@@ -59,8 +59,8 @@ __host__ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 // inside one super-square (16 + 16 panels) that the Infinity Cache holds.  An XCD whose queue
 // is exhausted steals from the next XCD's queue, so the tail stays balanced.
 struct Raster {
-    unsigned tilesPerDim;
-    unsigned squaresPerDim;
+    unsigned tileRows, tileCols;      // 256-point tiles along the queries / the candidates
+    unsigned squareCols;              // super-squares per row of super-squares
     unsigned long long perQueue;  // pops each queue serves
 };
 
@@ -72,22 +72,24 @@ constexpr int kCounterFound = 0;
 constexpr int kQueueBase = 16, kQueueStride = 16;  // queue heads sit on separate 128-byte lines
 constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
-__host__ __device__ inline Raster make_raster(long long n) {
+__host__ __device__ inline Raster make_raster(long long nQueries, long long nCandidates) {
     Raster r;
-    r.tilesPerDim = (unsigned)((n + kTile - 1) / kTile);
-    r.squaresPerDim = (r.tilesPerDim + kRaster - 1) / kRaster;
-    r.perQueue = (unsigned long long)r.squaresPerDim * r.squaresPerDim * kSubTiles;
+    r.tileRows = (unsigned)((nQueries + kTile - 1) / kTile);
+    r.tileCols = (unsigned)((nCandidates + kTile - 1) / kTile);
+    const unsigned squareRows = (r.tileRows + kRaster - 1) / kRaster;
+    r.squareCols = (r.tileCols + kRaster - 1) / kRaster;
+    r.perQueue = (unsigned long long)squareRows * r.squareCols * kSubTiles;
     return r;
 }
 
-// Pop t of queue q -> tile (row, col) in tile units.  Tiles outside the tilesPerDim grid are
+// Pop t of queue q -> tile (row, col) in tile units.  Tiles outside the tileRows x tileCols grid are
 // padding of the last super-squares: the caller skips them.
 __host__ __device__ inline void raster_decode(const Raster& r, unsigned q, unsigned long long t, unsigned* tr,
                                               unsigned* tc) {
     const unsigned long long sq = t / kSubTiles;
     const unsigned local = (unsigned)(t % kSubTiles);
-    *tr = (unsigned)(sq / r.squaresPerDim) * kRaster + (q >> 1) * kSubRows + local / kSubCols;
-    *tc = (unsigned)(sq % r.squaresPerDim) * kRaster + (q & 1) * kSubCols + local % kSubCols;
+    *tr = (unsigned)(sq / r.squareCols) * kRaster + (q >> 1) * kSubRows + local / kSubCols;
+    *tc = (unsigned)(sq % r.squareCols) * kRaster + (q & 1) * kSubCols + local % kSubCols;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -122,12 +124,15 @@ __global__ void reset_counters_kernel(unsigned long long* c) {
 
 // ------------------------------------------------------------------------------------------
 struct JoinParams {
-    const u32x4* pts;
-    long long ld16;  // row stride in 16-byte units
-    int n;
+    const u32x4* ptsQ;  // query rows
+    const u32x4* ptsC;  // candidate rows (the same buffer for a self-join)
+    long long ldQ16, ldC16;  // row strides in 16-byte units
+    int nQ, nC;
+    int selfJoin;  // queries and candidates are the same set: (i, i) is always a pair
     int nSlabs;
     float eps2;
-    const float* sums;
+    const float* sumsQ;
+    const float* sumsC;
     unsigned long long* counters;
     int2* pairs;
     unsigned long long cap;
@@ -144,13 +149,13 @@ struct JoinParams {
 // wave-wide (its result is the ballot), and only blocks in which some lane has a candidate evaluate
 // the reference formula exactly:  (s_q + s_c) - 2*acc <= eps^2  in FP32 (source/warpMma.cuh:241-257).
 //
-// kEdge: the tile touches the diagonal or the ragged end of the dataset; every block is evaluated
-// exactly, self pairs are forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
+// kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; every block is
+// evaluated exactly, self pairs are forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
 // Returns per-lane hit bits: mask[fi/2] bit ((fi&1)*16 + fj*4 + r).
 template <bool kEdge>
 __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const float* sQ,
                                            const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
-                                           int quad, int n, float eps2, float margin,
+                                           int quad, int nQ, int nC, int selfJoin, float eps2, float margin,
                                            unsigned (&mask)[kFragRows / 2]) {
     float thr[kFragCols];
 #pragma unroll
@@ -178,7 +183,7 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
                         bool hit = d2 <= eps2;
                         if (kEdge) {
                             const int q = qBase + fi * 16 + quad * 4 + r;
-                            hit = (hit || q == cand[fj]) && q < n && cand[fj] < n;
+                            hit = (hit || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
                         }
                         m = hit ? (m | (1u << (h * 16 + fj * 4 + r))) : m;
                     }
@@ -264,7 +269,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     while (ticket != kDone) {
         unsigned tr, tc;
         raster_decode(p.raster, (unsigned)(ticket / p.raster.perQueue), ticket % p.raster.perQueue, &tr, &tc);
-        if (tr >= p.raster.tilesPerDim || tc >= p.raster.tilesPerDim) {  // padding tile of the raster
+        if (tr >= p.raster.tileRows || tc >= p.raster.tileCols) {  // padding tile of the raster
             __syncthreads();
             if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
             __syncthreads();
@@ -274,21 +279,21 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
 
         // rows past the end of the dataset re-read the last real row; their results are masked
-        const char* const gA = reinterpret_cast<const char*>(p.pts + (long long)rowBase * p.ld16);
-        const char* const gB = reinterpret_cast<const char*>(p.pts + (long long)colBase * p.ld16);
+        const char* const gA = reinterpret_cast<const char*>(p.ptsQ + (long long)rowBase * p.ldQ16);
+        const char* const gB = reinterpret_cast<const char*>(p.ptsC + (long long)colBase * p.ldC16);
         unsigned offA[4], offB[4];  // byte offsets from the tile's first row
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = cpRow0 + 8 * i;
             const int chunk = (lane & 7) ^ swz(r);
-            offA[i] = (unsigned)(min(r, p.n - 1 - rowBase) * (int)p.ld16 + chunk) * 16u;
-            offB[i] = (unsigned)(min(r, p.n - 1 - colBase) * (int)p.ld16 + chunk) * 16u;
+            offA[i] = (unsigned)(min(r, p.nQ - 1 - rowBase) * (int)p.ldQ16 + chunk) * 16u;
+            offB[i] = (unsigned)(min(r, p.nC - 1 - colBase) * (int)p.ldC16 + chunk) * 16u;
         }
         {
             // squared norms of the tile's 256 queries and 256 candidates, plus their maximum
             // (it scales the safety margin of the epilogue's screening test)
-            const float mySum = tid < kTile ? p.sums[min(rowBase + tid, p.n - 1)]
-                                            : p.sums[min(colBase + tid - kTile, p.n - 1)];
+            const float mySum = tid < kTile ? p.sumsQ[min(rowBase + tid, p.nQ - 1)]
+                                            : p.sumsC[min(colBase + tid - kTile, p.nC - 1)];
             sQ[tid] = mySum;  // sC == sQ + kTile
             float m = __builtin_fabsf(mySum);
 #pragma unroll
@@ -388,16 +393,18 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
             }
             // margin of the screening test: covers the FP32 roundings of both forms of the inequality
-            const bool edge = (tr == tc) || rowBase + kTile > p.n || colBase + kTile > p.n;
+            const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
             float sMax = sWaveMax[0];
 #pragma unroll
             for (int w = 1; w < 8; ++w) sMax = __builtin_fmaxf(sMax, sWaveMax[w]);
             const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
             unsigned mask[kFragRows / 2];
             if (edge)
-                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, margin, mask);
+                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
+                                 mask);
             else
-                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.n, p.eps2, margin, mask);
+                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
+                                  mask);
 
             int mine = 0;
 #pragma unroll
@@ -465,26 +472,26 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
 }  // namespace
 
-unsigned long long raster_count(long long n) { return make_raster(n).perQueue * kQueues; }
+unsigned long long raster_count(long long nQ, long long nC) { return make_raster(nQ, nC).perQueue * kQueues; }
 
 // Index idx enumerates the queues round-robin: queue idx % 8, position idx / 8 -- the order in
 // which eight equally fast XCDs would take the tiles.  Returns 0 past the end, 2 for a padding
 // tile that the kernel skips, 1 for a real tile.
-int raster_coord(unsigned long long idx, long long n, int* row, int* col) {
-    const Raster r = make_raster(n);
+int raster_coord(unsigned long long idx, long long nQ, long long nC, int* row, int* col) {
+    const Raster r = make_raster(nQ, nC);
     if (idx >= r.perQueue * kQueues) return 0;
     unsigned tr, tc;
     raster_decode(r, (unsigned)(idx % kQueues), idx / kQueues, &tr, &tc);
     *row = (int)tr * kTile;
     *col = (int)tc * kTile;
-    return (tr < r.tilesPerDim && tc < r.tilesPerDim) ? 1 : 2;
+    return (tr < r.tileRows && tc < r.tileCols) ? 1 : 2;
 }
 
 int counter_words() { return kCounterWords; }
 
-unsigned long long tile_count(long long n) {
-    const Raster r = make_raster(n);
-    return (unsigned long long)r.tilesPerDim * r.tilesPerDim;
+unsigned long long tile_count(long long nQ, long long nC) {
+    const Raster r = make_raster(nQ, nC);
+    return (unsigned long long)r.tileRows * r.tileCols;
 }
 
 int lds_chunk_slot(int row, int chunk) { return (chunk ^ swz(row)) & 7; }
@@ -526,17 +533,22 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
         configured = true;
     }
     JoinParams p;
-    p.pts = static_cast<const u32x4*>(l.points);
-    p.ld16 = l.ld / 8;
-    p.n = l.n;
+    p.ptsQ = static_cast<const u32x4*>(l.queries);
+    p.ptsC = static_cast<const u32x4*>(l.candidates);
+    p.ldQ16 = l.ldQ / 8;
+    p.ldC16 = l.ldC / 8;
+    p.nQ = l.nQ;
+    p.nC = l.nC;
+    p.selfJoin = l.selfJoin ? 1 : 0;
     p.nSlabs = l.dPad / kSlabK;
     p.eps2 = l.eps2;
-    p.sums = l.sums;
+    p.sumsQ = l.sumsQ;
+    p.sumsC = l.sumsC;
     p.counters = l.counters;
     p.pairs = static_cast<int2*>(l.pairs);
     p.cap = l.cap;
-    p.raster = make_raster(l.n);
-    unsigned long long realTiles = (unsigned long long)p.raster.tilesPerDim * p.raster.tilesPerDim;
+    p.raster = make_raster(l.nQ, l.nC);
+    unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
     unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
     if (l.epilogue)

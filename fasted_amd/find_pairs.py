@@ -112,6 +112,10 @@ def load_findpairs(path: str = None):
     lib.fasted_self_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_double, c.c_void_p,
                                             c.c_void_p, c.c_ulonglong, c.c_uint, c.c_void_p,
                                             c.POINTER(FastedJoinStats)]
+    lib.fasted_join_device.restype = c.c_int
+    lib.fasted_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_longlong, c.c_void_p, c.c_longlong, c.c_longlong,
+                                       c.c_int, c.c_double, c.c_void_p, c.c_void_p, c.c_void_p, c.c_ulonglong, c.c_uint,
+                                       c.c_void_p, c.POINTER(FastedJoinStats)]
     lib.fasted_sum_squared_device.restype = c.c_int
     lib.fasted_sum_squared_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_void_p, c.c_void_p]
     lib.fasted_raster_coord.restype = c.c_int
@@ -205,6 +209,16 @@ def find_epsilon(target_selectivity, initial_epsilon=0.0):
     _check(lib, lib.fasted_find_epsilon(float(target_selectivity), float(initial_epsilon), ctypes.byref(eps),
                                         ctypes.byref(sel), ctypes.byref(probes)))
     return eps.value, sel.value, probes.value
+
+
+def join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates, d, epsilon, pairs_ptr,
+                cap, flags=FASTED_SORT_PAIRS, stream=None):
+    """Join of two different point sets on raw device pointers; returns FastedJoinStats."""
+    lib = load_findpairs()
+    st = FastedJoinStats()
+    _check(lib, lib.fasted_join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates,
+                                       d, float(epsilon), None, None, pairs_ptr, cap, flags, stream, ctypes.byref(st)))
+    return st
 
 
 def sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream=None):

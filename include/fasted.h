@@ -108,6 +108,17 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
                             FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
                             FastedJoinStats* stats);
 
+/* Join of two different sets: every pair (q, c), q indexing the queries and c the candidates, with
+ * dist <= epsilon; no pair is forced (there are no self pairs).  Same buffer rules per set as
+ * fasted_self_join_device.  The reference's device parameters already carry distinct query and
+ * candidate pointers (source/findPairs.cuh:90-100) although its host code always passes one set twice
+ * (source/findPairs.cuh:619); joining a dataset block by block through this entry is how a dataset
+ * larger than the device memory would be handled. */
+int fasted_join_device(const void* d_queries, long long n_queries, long long ld_queries, const void* d_candidates,
+                       long long n_candidates, long long ld_candidates, int d, double epsilon, float* d_sums_queries,
+                       float* d_sums_candidates, FastedPair* d_pairs, unsigned long long cap, unsigned flags,
+                       void* stream, FastedJoinStats* stats);
+
 /* Squared norms only: sums[i] = sum_k x_ik^2 in FP32.  Replaces
  * SumSqd::ComputeSquaredSums (source/sumSquared.cuh:84-118). */
 int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream);

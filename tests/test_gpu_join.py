@@ -190,3 +190,34 @@ def test_rerun_changes_epsilon_on_resident_data(fasted):
     assert r1.pairsFound > r0.pairsFound
     assert r0.TFLOPS > 0 and r0.totalTime > 0
     lib.releaseResources()
+
+
+@pytest.mark.parametrize("nq,nc,d", [(300, 1000, 64), (1000, 300, 128), (257, 5000, 192), (4100, 513, 64)])
+def test_two_set_join_matches_the_checker(fasted, nq, nc, d):
+    """Queries and candidates from different sets (no forced pairs).  Checked by running the
+    checker's self-join on the stacked sets and keeping the (query, candidate) block."""
+    import torch
+
+    both = datasets.uniform_bytes(nq + nc, d, seed=nq + nc)
+    # plant exact duplicates across the two sets: distance 0 pairs must be found, none is forced
+    both[nq + 5] = both[3]
+    both[nq + 17] = both[nq - 1]
+    eps = datasets.epsilon_for_neighbours(both, 6)
+    q = torch.from_numpy(both[:nq].view(np.int16).copy()).cuda()
+    c = torch.from_numpy(both[nq:].view(np.int16).copy()).cuda()
+    cap = 200 * (nq + nc)
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    st = fasted.join_device(q.data_ptr(), nq, d, c.data_ptr(), nc, d, d, eps, pairs.data_ptr(), cap)
+    got = pairs[: st.pairsStored].cpu().numpy()
+    assert st.pairsFound == st.pairsStored
+    stacked = oracle.self_join_f64(both, eps)
+    block = stacked[(stacked[:, 0] < nq) & (stacked[:, 1] >= nq)].copy()
+    block[:, 1] -= nq
+    stats, diff, side = oracle.pair_stats(got, block, want_diff=True)
+    # disagreements only inside the band (distances from the stacked data: shift the candidate index back)
+    shifted = diff.copy()
+    shifted[:, 1] += nq
+    dist = oracle.pair_distances_f64(both, shifted)
+    assert np.all(np.abs(dist - eps) / eps <= 1e-3), (stats, dist)
+    assert {(3, 5), (nq - 1, 17)} <= {tuple(p) for p in got}
+    assert stats["both"] > 0
