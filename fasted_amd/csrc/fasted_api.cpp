@@ -283,14 +283,14 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
 }
 
 // Shared body of the three run entry points, the counterpart of run() in
-// source/main.cu:198-248: failures are printed and end the process, as there.
-Results run_source(fasted::PointSource* src, double epsilon, bool savePairs) {
+// source/main.cu:198-248: failures are printed and end the process, as there.  `fresh` is a newly
+// built dataset that becomes the resident one; without it the resident dataset is reused (reRun).
+Results run_resident(fasted::PointTable* fresh, double epsilon, bool savePairs) {
     try {
         std::string name;
-        if (src) {
-            name = src->name();
-            if (!quiet()) std::cout << "Building point list" << std::endl;
-            g_res.table = fasted::build_point_table(*src, fasted::kSlabK, fasted::kTile);
+        if (fresh) {
+            name = fresh->name;
+            g_res.table = std::move(*fresh);
             g_res.uploaded = false;
             if (!quiet()) {
                 std::cout << "Number of points is: " << g_res.table.n << std::endl;
@@ -303,11 +303,24 @@ Results run_source(fasted::PointSource* src, double epsilon, bool savePairs) {
                       << std::endl;
             std::cout << "Input Search Dimensions:\nM: " << tb.n << "\nN: " << tb.n << "\nK: " << tb.d << std::endl;
         }
-        return find_pairs_resident(epsilon, savePairs, src == nullptr, name);
+        return find_pairs_resident(epsilon, savePairs, fresh == nullptr, name);
     } catch (const std::exception& e) {
         std::cout << "Error: Failed to run. " << e.what() << std::endl;
         std::exit(EXIT_FAILURE);
     }
+}
+
+template <typename Build>
+Results run_built(Build&& build, double epsilon, bool savePairs) {
+    fasted::PointTable table;
+    try {
+        if (!quiet()) std::cout << "Building point list" << std::endl;
+        table = build();
+    } catch (const std::exception& e) {
+        std::cout << "Error: Failed to run. " << e.what() << std::endl;
+        std::exit(EXIT_FAILURE);
+    }
+    return run_resident(&table, epsilon, savePairs);
 }
 
 // Uploads the resident dataset if it is not on the device yet.
@@ -359,23 +372,23 @@ extern "C" {
 Results runFromExponentialDataset(int size, int dimensionality, double lambda, double max, double epsilon,
                                   bool savePairs) {
     if (!quiet()) std::cout << "Running from a generated exponential dataset" << std::endl;
-    fasted::ExponentialSource src(size, dimensionality, lambda, max);
-    return run_source(&src, epsilon, savePairs);
+    return run_built(
+        [&] {
+            fasted::ExponentialSource src(size, dimensionality, lambda, max);
+            return fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+        },
+        epsilon, savePairs);
 }
 
 Results runFromFile(const char* filename, double epsilon, bool savePairs) {
-    try {
-        const std::string path(filename ? filename : "");
-        if (!quiet()) std::cout << "Running from file: " << path << std::endl;
-        fasted::CsvSource src(path, ',');
-        return run_source(&src, epsilon, savePairs);
-    } catch (const std::exception& e) {  // the reference lets a missing file terminate the process
-        std::cout << "Error: Failed to run. " << e.what() << std::endl;
-        std::exit(EXIT_FAILURE);
-    }
+    const std::string path(filename ? filename : "");
+    if (!quiet()) std::cout << "Running from file: " << path << std::endl;
+    // a missing file ends the process here as it does in the reference
+    return run_built([&] { return fasted::load_csv_table(path, ',', fasted::kSlabK, fasted::kTile); }, epsilon,
+                     savePairs);
 }
 
-Results reRun(double epsilon, bool savePairs) { return run_source(nullptr, epsilon, savePairs); }
+Results reRun(double epsilon, bool savePairs) { return run_resident(nullptr, epsilon, savePairs); }
 
 void releaseResources(void) {
     g_res.drop_device();
@@ -459,9 +472,10 @@ int fasted_load_exponential_dataset(int size, int dimensionality, double lambda,
 
 int fasted_load_file(const char* filename) {
     return guarded([&] {
-        fasted::CsvSource src(std::string(filename ? filename : ""), ',');
+        fasted::PointTable table = fasted::load_csv_table(std::string(filename ? filename : ""), ',', fasted::kSlabK,
+                                                          fasted::kTile);
         g_res.drop_device();
-        g_res.table = fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+        g_res.table = std::move(table);
     });
 }
 

@@ -253,3 +253,54 @@ def test_pair_statistics_and_per_point_iou():
     assert (s.both_sides, s.right_only, s.left_only) == (o["both"], o["right_only"], o["left_only"])
     iou = ex.per_point_iou([[0, 0], [0, 1], [1, 1], [2, 2]], [[0, 0], [0, 2], [1, 1]], 4)
     assert iou.tolist() == [1 / 3, 1.0, 0.0, 1.0]
+
+
+def test_csv_loader_multithreaded_equals_numpy_parse(lib, tmp_path, monkeypatch):
+    rng = np.random.default_rng(12)
+    vals = rng.exponential(1 / 40.0, (5003, 37))
+    path = tmp_path / "big.csv"
+    with open(path, "w") as f:
+        for i, row in enumerate(vals):
+            sep = ",  " if i % 7 == 0 else ","  # leading blanks are skipped like std::stod does
+            f.write(sep.join(repr(float(v)) for v in row) + ("\r\n" if i % 11 == 0 else "\n"))
+    want = oracle.quantize(vals)
+    for threads in ("1", "3", "16"):
+        monkeypatch.setenv("FASTED_CSV_THREADS", threads)
+        assert lib.fasted_load_file(str(path).encode()) == 0
+        bits, n, d, name = fasted_amd.resident_points()
+        assert (n, d, name) == (5003, 37, "big") and bits.shape == (5120, 64)
+        assert np.array_equal(bits[:n, :d], want) and bits[n:].sum() == 0 and bits[:, d:].sum() == 0
+    # the first bad line wins, whichever thread meets it
+    lines = open(path).read().split("\n")
+    lines[4000] = "1,2,3"
+    lines[900] = lines[900].replace(",", ",oops,", 1)
+    bad = tmp_path / "bad.csv"
+    bad.write_text("\n".join(lines))
+    assert lib.fasted_load_file(str(bad).encode()) != 0
+    assert lib.fasted_last_error() == b"stod"
+    no_newline = tmp_path / "nonl.csv"
+    no_newline.write_text("1,2\n3,4")  # last line without a newline still counts
+    assert lib.fasted_load_file(str(no_newline).encode()) == 0
+    assert fasted_amd.resident_points()[1] == 2
+    blank = tmp_path / "blank.csv"
+    blank.write_text("1,2\n\n3,4\n")  # an empty line is a point with no dimensions
+    assert lib.fasted_load_file(str(blank).encode()) != 0
+    assert lib.fasted_last_error().decode() == GOLDEN["ragged_error"]
+
+
+def test_host_quantisation_rounds_twice_like_the_reference(lib, tmp_path):
+    """double -> float -> half is not double -> half: doubles whose float image is an exact tie between
+    two halves round differently.  The loader must take the two-step route (PointListBuilder.hpp:57-73)."""
+    rng = np.random.default_rng(99)
+    x = rng.exponential(1 / 40.0, 4_000_000)
+    two_step = x.astype(np.float32).astype(np.float16).view(np.uint16)
+    one_step = x.astype(np.float16).view(np.uint16)
+    tricky = np.concatenate([[0.01198196413320991], x[two_step != one_step][:63]])
+    assert len(tricky) >= 8
+    path = tmp_path / "ties.csv"
+    path.write_text("\n".join(repr(float(v)) for v in tricky) + "\n")
+    assert lib.fasted_load_file(str(path).encode()) == 0
+    bits, n, d, _ = fasted_amd.resident_points()
+    assert (n, d) == (len(tricky), 1)
+    assert np.array_equal(bits[:n, 0], tricky.astype(np.float32).astype(np.float16).view(np.uint16))
+    assert np.array_equal(bits[:n, 0], oracle.quantize(tricky))
