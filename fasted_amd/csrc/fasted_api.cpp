@@ -142,6 +142,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.nQ = (int)q.n;
     jl.nC = (int)c.n;
     jl.selfJoin = selfJoin;
+    jl.symmetric = selfJoin && (flags & FASTED_SYMMETRIC);
     jl.dPad = dPad;
     jl.eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
     jl.sumsQ = sumsQ;

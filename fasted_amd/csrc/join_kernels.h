@@ -16,6 +16,7 @@ struct JoinLaunch {
     long long ldQ, ldC;          // row strides in halves (multiples of 8)
     int nQ, nC;                  // real points
     bool selfJoin;               // same set on both sides: (i, i) always counts as a pair
+    bool symmetric;              // self-join: only tiles on/above the diagonal are computed, pairs mirrored
     int dPad;                    // K extent, multiple of kSlabK
     float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
     const float* sumsQ;          // squared norms of the queries

@@ -129,6 +129,7 @@ struct JoinParams {
     long long ldQ16, ldC16;  // row strides in 16-byte units
     int nQ, nC;
     int selfJoin;  // queries and candidates are the same set: (i, i) is always a pair
+    int symmetric; // self-join only: compute tiles on and above the diagonal, emit (q,c) and (c,q)
     int nSlabs;
     float eps2;
     const float* sumsQ;
@@ -269,7 +270,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     while (ticket != kDone) {
         unsigned tr, tc;
         raster_decode(p.raster, (unsigned)(ticket / p.raster.perQueue), ticket % p.raster.perQueue, &tr, &tc);
-        if (tr >= p.raster.tileRows || tc >= p.raster.tileCols) {  // padding tile of the raster
+        // padding tile of the raster, or a tile below the diagonal whose pairs its mirror tile emits
+        if (tr >= p.raster.tileRows || tc >= p.raster.tileCols || (p.symmetric && tc < tr)) {
             __syncthreads();
             if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
             __syncthreads();
@@ -406,9 +408,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
                                   mask);
 
+            // symmetric mode: a tile above the diagonal also stands for its mirror image
+            const bool mirror = p.symmetric && tr != tc;
             int mine = 0;
 #pragma unroll
             for (int fp = 0; fp < kFragRows / 2; ++fp) mine += __builtin_popcount(mask[fp]);
+            if (mirror) mine *= 2;
             if (__builtin_amdgcn_ballot_w64(mine != 0) != 0ull) {
                 // wave-level compaction: inclusive prefix sum of per-lane counts, one reservation
                 int incl = mine;
@@ -440,13 +445,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         const int fi = fp * 2 + (bit >> 4), fj = (bit >> 2) & 3, r = bit & 3;
                         const int q = qBase + fi * 16 + quad * 4 + r;
                         const int c = colBase + wc * kWaveCols + fj * 16 + l16;
-                        if (idx < fit) {
-                            sStage[pos + idx] = make_int2(q, c);
-                        } else {
-                            const unsigned long long slot = gbase + (idx - fit);
-                            if (slot < p.cap) p.pairs[slot] = make_int2(q, c);
-                        }
-                        ++idx;
+                        auto put = [&](unsigned at, int first, int second) {
+                            if (at < fit) {
+                                sStage[pos + at] = make_int2(first, second);
+                            } else {
+                                const unsigned long long slot = gbase + (at - fit);
+                                if (slot < p.cap) p.pairs[slot] = make_int2(first, second);
+                            }
+                        };
+                        put(idx++, q, c);
+                        if (mirror) put(idx++, c, q);
                     }
                 }
             }
@@ -540,6 +548,7 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
     p.nQ = l.nQ;
     p.nC = l.nC;
     p.selfJoin = l.selfJoin ? 1 : 0;
+    p.symmetric = (l.selfJoin && l.symmetric) ? 1 : 0;
     p.nSlabs = l.dPad / kSlabK;
     p.eps2 = l.eps2;
     p.sumsQ = l.sumsQ;

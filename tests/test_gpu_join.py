@@ -221,3 +221,18 @@ def test_two_set_join_matches_the_checker(fasted, nq, nc, d):
     assert np.all(np.abs(dist - eps) / eps <= 1e-3), (stats, dist)
     assert {(3, 5), (nq - 1, 17)} <= {tuple(p) for p in got}
     assert stats["both"] > 0
+
+
+@pytest.mark.parametrize("n,d", [(700, 64), (2048, 128), (5000, 192)])
+def test_symmetric_option_gives_the_same_pair_set(fasted, n, d):
+    """FASTED_SYMMETRIC computes only the tiles on and above the diagonal and mirrors the pairs: the
+    sorted pair list must be identical to the default full computation."""
+    from fasted_amd import find_pairs as fp
+
+    bits = datasets.uniform_bytes(n, d, seed=3 * n + d)
+    eps = datasets.epsilon_for_neighbours(bits, 12)
+    full, st_full, _ = device_join(fasted, bits, eps)
+    half, st_half, _ = device_join(fasted, bits, eps, flags=fp.FASTED_SORT_PAIRS | fp.FASTED_SYMMETRIC)
+    assert st_half.pairsFound == st_full.pairsFound
+    assert np.array_equal(half, full)
+    check_against_fp64(bits, n, eps, half)
