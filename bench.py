@@ -255,6 +255,8 @@ def main():
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": traffic, "traffic_detail": traffic_detail},
     }
+    if not args.no_epilogue and st.pairsStored == st.pairsFound:
+        out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
     if not args.no_epilogue:
         # Not part of `value`: the opt-in FASTED_SYMMETRIC mode computes only the tiles on and above the
         # diagonal (same pair set).  Its rate is 2*N^2*D over its time, i.e. an *effective* figure: the
@@ -266,10 +268,6 @@ def main():
             "ms_per_step": sym_ms, "effective_tflops": flops / (sym_ms / 1000.0) / 1e12,
             "pairs_found": int(sym.pairsFound), "same_pair_count": bool(sym.pairsFound == st.pairsFound),
             "note": "opt-in, not the headline: about half of 2*N^2*D is actually executed"}
-        # leave the default run's pairs in the buffer for the parity check below
-        st = step()
-    if not args.no_epilogue and st.pairsStored == st.pairsFound:
-        out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
     print(json.dumps(out))
