@@ -180,6 +180,8 @@ def main():
     ap.add_argument("--eps", type=float, default=0.0, help="skip calibration and use this epsilon")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogue", action="store_true", help="measurement: contraction only")
+    ap.add_argument("--no-symmetric-option", action="store_true",
+                    help="skip the extra launch that measures the opt-in FASTED_SYMMETRIC mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 1 GiB read + 1 GiB write elementwise kernel (to scale FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -257,7 +259,7 @@ def main():
     }
     if not args.no_epilogue and st.pairsStored == st.pairsFound:
         out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
-    if not args.no_epilogue:
+    if not args.no_epilogue and not args.no_symmetric_option:
         # Not part of `value`: the opt-in FASTED_SYMMETRIC mode computes only the tiles on and above the
         # diagonal (same pair set).  Its rate is 2*N^2*D over its time, i.e. an *effective* figure: the
         # matrix cores execute about half of those FLOPs.
