@@ -75,7 +75,7 @@ def calibrate_epsilon(torch, pts, neighbours, sample=4096, seed=4242):
     qs = (q * q).sum(1)
     k = int(round(neighbours * m)) + m + 1  # + the m self pairs
     best = torch.full((0,), float("inf"), device="cuda")
-    chunk = max(1, min(n, (1 << 27) // d))
+    chunk = max(1, min(n, (1 << 27) // d, (1 << 30) // m))  # torch.topk sorts at most INT_MAX elements
     for c0 in range(0, n, chunk):
         c = pts[c0:c0 + chunk].to(torch.float32)
         d2 = qs[:, None] + (c * c).sum(1)[None, :] - 2.0 * (q @ c.T)
@@ -215,7 +215,7 @@ def main():
     if args.n or args.d:
         label = f"{kind} {n}x{d} (override of {args.config})"
     pts = generate_points(torch, kind, n, d, seed=20260 + n % 997)
-    eps = args.eps or calibrate_epsilon(torch, pts, neighbours, sample=16384 if n >= 500_000 else 4096)
+    eps = args.eps or calibrate_epsilon(torch, pts, neighbours, sample=16384 if n >= 500_000 and neighbours <= 100 else 4096)
     # pair buffer: the reference's N*256 records, or 1.25x the expected count when that is larger
     cap = int(max(n * 256, 1.25 * n * (neighbours + 1)))
     pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")

@@ -3,19 +3,27 @@
 //   sum_squared_kernel   FP32 squared norm of every FP16 point; HBM-bound, 16-byte
 //                        coalesced loads, lane-group shuffle reduction.  Stands where the
 //                        reference has SumSqd::SquaredSumsKernel (source/sumSquared.cuh:53-73).
-//   join_kernel          persistent workgroups pull 256x256 tiles of the N x N distance
-//                        matrix from an atomic work queue (the reference's on-demand
-//                        rasterizer, source/rasterizer/onDemandRasterizer.cuh:78-108), form
-//                        Q.C^T with v_mfma_f32_32x32x16_f16 from XOR-swizzled, double-buffered
-//                        LDS slabs (source/findPairs.cuh:360-546 is the reference's kernel),
-//                        and run the fused test  (s_q + s_c) - 2 q.c <= eps^2
-//                        (source/warpMma.cuh:220-273) with wave-level compaction: one
-//                        atomic reservation per wave instead of one per pair
-//                        (source/pair.cuh:123-133).
+//   join_kernel          persistent workgroups pull 256x256 tiles of the distance matrix from
+//                        per-XCD atomic work queues (the reference's on-demand rasterizer,
+//                        source/rasterizer/onDemandRasterizer.cuh:78-108), form Q.C^T with
+//                        v_mfma_f32_16x16x32_f16 from XOR-swizzled, double-buffered LDS slabs that
+//                        global_load_lds_dwordx4 fills without passing through registers
+//                        (source/findPairs.cuh:360-546 is the reference's kernel), and run the
+//                        fused test  (s_q + s_c) - 2 q.c <= eps^2  (source/warpMma.cuh:220-273)
+//                        with wave-level compaction into an LDS staging area: one global
+//                        reservation per workgroup flush instead of two atomics per pair
+//                        (source/pair.cuh:123-133).  The first slab and the squared norms of the
+//                        next tile travel during the last slab and the epilogue of the current one.
 //
 // Data layout: points are row-major FP16, one point per row, row stride `ld` halves.  Both
 // MFMA operands are "row = point, 8 consecutive k per lane", so the query tile and the
 // candidate tile are staged in LDS in the same [256 rows][64 halves] form.
+//
+// The kernel is written so that it needs no scratch memory: a scratch reload in the epilogue would
+// have to wait for every outstanding vector-memory operation of the wave, i.e. for the transfers of
+// the next tile that are meant to stay in flight there.  Build with
+// -mllvm -amdgpu-atomic-optimizer-strategy=None: the queue reservation is made by one lane a whole
+// tile before its result is used, and the optimiser's wave-reduction form would wait for it on the spot.
 #include "join_kernels.h"
 
 #include <type_traits>
@@ -31,10 +39,10 @@ constexpr int kThreads = 512;                       // 8 waves: 2 (rows) x 4 (co
 constexpr int kRowBytes = kSlabK * 2;               // one LDS row of a slab: 128 B = 8 chunks of 16 B
 constexpr int kOperandBytes = kTile * kRowBytes;    // 32 KiB per operand per stage
 constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 64 KiB
-constexpr int kLdsSums = 2 * kStageBytes;           // s_q[256] then s_c[256]
-constexpr int kLdsNext = kLdsSums + 2 * kTile * 4;  // next queue index
-constexpr int kLdsWaveMax = kLdsNext + 16;          // per-wave max of the tile's squared norms
-constexpr int kLdsStageCount = kLdsWaveMax + 8 * 4; // pairs waiting in the LDS staging area (u32) + flush base (u64)
+constexpr int kLdsSums = 2 * kStageBytes;           // two buffers of s_q[256] then s_c[256] (current / next tile)
+constexpr int kSumsBytes = 2 * kTile * 4;
+constexpr int kLdsNext = kLdsSums + 2 * kSumsBytes; // next tile of this workgroup: (row, col) as two u32
+constexpr int kLdsStageCount = kLdsNext + 16;       // pairs waiting in the LDS staging area (u32) + flush base (u64)
 constexpr int kLdsStage = kLdsStageCount + 16;      // staged pairs
 constexpr int kStagePairs = 3072;                   // 24 KiB of 8-byte records
 constexpr int kLdsBytes = kLdsStage + kStagePairs * 8;
@@ -152,7 +160,8 @@ struct JoinParams {
 //
 // kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; every block is
 // evaluated exactly, self pairs are forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
-// Returns per-lane hit bits: mask[fi/2] bit ((fi&1)*16 + fj*4 + r).
+// Returns per-lane hit bits, shifted in from the right in evaluation order: element e = (fi&1)*16 + fj*4 + r
+// of the pair of row blocks fi/2 ends up in bit 31 - e of mask[fi/2].
 template <bool kEdge>
 __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const float* sQ,
                                            const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
@@ -186,8 +195,10 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
                             const int q = qBase + fi * 16 + quad * 4 + r;
                             hit = (hit || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
                         }
-                        m = hit ? (m | (1u << (h * 16 + fj * 4 + r))) : m;
+                        m = (m << 1) | (hit ? 1u : 0u);
                     }
+                } else {
+                    m <<= 4;
                 }
             }
         }
@@ -195,54 +206,73 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
     }
 }
 
+// Lane number 0..63, re-derived from the execution mask where it is needed.  Volatile on purpose: the
+// optimiser then cannot hoist it (and what is derived from it) out of the tile loop, where it would
+// occupy registers, or spill, across the k loop.
+__device__ __forceinline__ int lane_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 template <bool kEpilogue>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
-    extern __shared__ __align__(16) unsigned char lds[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+    __shared__ __align__(16) unsigned char lds[kLdsBytes];
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);  // wave-uniform, lives in an SGPR
     const int wr = wave >> 2, wc = wave & 3;
-    const int l16 = lane & 15, quad = lane >> 4;
-
-    // copy role: global -> LDS without passing through registers (global_load_lds_dwordx4).
-    // One wave instruction fills 1 KiB of LDS = 8 rows of a slab, lane l landing in row l/8,
-    // chunk slot l%8; the swizzle is applied on the global side by choosing which 16-byte
-    // chunk of the row each lane fetches, so the 8 lanes of a row still read one 128-byte line.
-    // Wave w owns rows [32w, 32w+32) of both operands: 4 instructions each.
-    const int cpRow0 = wave * 32 + (lane >> 3);
 
     // fragment role (v_mfma_f32_16x16x32_f16): lane reads row l%16 of a 16-row block and the
     // 8 halves k = 8*(l/16) .. +7 of a 32-wide k-step, i.e. chunk 4*ks + l/16 of the slab row.
     int aOff[2], bOff[2];
+    {
+        const int lane = lane_now();
+        const int l16 = lane & 15, quad = lane >> 4;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        const int slot = ((ks * 4 + quad) ^ swz(l16)) << 4;
-        aOff[ks] = (wr * kWaveRows + l16) * kRowBytes + slot;
-        bOff[ks] = kOperandBytes + (wc * kWaveCols + l16) * kRowBytes + slot;
+        for (int ks = 0; ks < 2; ++ks) {
+            const int slot = ((ks * 4 + quad) ^ swz(l16)) << 4;
+            aOff[ks] = (wr * kWaveRows + l16) * kRowBytes + slot;
+            bOff[ks] = kOperandBytes + (wc * kWaveCols + l16) * kRowBytes + slot;
+        }
     }
 
-    float* const sQ = reinterpret_cast<float*>(lds + kLdsSums);
-    float* const sC = sQ + kTile;
-    unsigned long long* const sNext = reinterpret_cast<unsigned long long*>(lds + kLdsNext);
-    float* const sWaveMax = reinterpret_cast<float*>(lds + kLdsWaveMax);
+    // LDS byte address of lds[0], for the LDS instructions written out by hand below
+    const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // next tile: [0] row, [1] col
     unsigned* const sStageCount = reinterpret_cast<unsigned*>(lds + kLdsStageCount);
     unsigned long long* const sFlushBase = reinterpret_cast<unsigned long long*>(lds + kLdsStageCount + 8);
     int2* const sStage = reinterpret_cast<int2*>(lds + kLdsStage);
 
     // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
     const unsigned home = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (kQueues - 1);
+    constexpr unsigned kNoTile = ~0u;
 
-    // A ticket is queue * perQueue + position; kDone means every queue is exhausted.
-    const unsigned long long kDone = ~0ull;
-    auto take = [&](unsigned firstQueue, unsigned long long firstPos) -> unsigned long long {
-        // firstPos was already popped from firstQueue; on exhaustion move on to the other queues
-        unsigned q = firstQueue;
-        unsigned long long pos = firstPos;
-        for (int tries = 0; tries < kQueues; ++tries) {
-            if (pos < p.raster.perQueue) return (unsigned long long)q * p.raster.perQueue + pos;
-            q = (q + 1) & (kQueues - 1);
-            if (tries + 1 < kQueues) pos = atomicAdd(&p.counters[kQueueBase + q * kQueueStride], 1ull);
+    // Thread 0 only.  `pos` was popped from the home queue; walks on (and on to the other queues
+    // once a queue is exhausted) until a tile that has to be computed turns up.  Skipped on the way:
+    // padding tiles of the last super-squares and, in symmetric mode, tiles below the diagonal.
+    auto find_tile = [&](unsigned long long pos, unsigned* row, unsigned* col) {
+        // the divisors pass through an empty volatile statement so that the reciprocals the division
+        // needs are formed here, once per tile, instead of living in registers across the k loop
+        Raster ras = p.raster;
+        asm volatile("" : "+s"(ras.squareCols));
+        unsigned q = home;
+        int hops = 0;
+        *row = kNoTile;
+        *col = 0u;
+        for (;;) {
+            if (pos < ras.perQueue) {
+                unsigned tr, tc;
+                raster_decode(ras, q, pos, &tr, &tc);
+                if (tr < ras.tileRows && tc < ras.tileCols && !(p.symmetric && tc < tr)) {
+                    *row = tr;
+                    *col = tc;
+                    return;
+                }
+            } else {
+                if (++hops == kQueues) return;  // every queue is exhausted
+                q = (q + 1) & (kQueues - 1);
+            }
+            pos = atomicAdd(&p.counters[kQueueBase + q * kQueueStride], 1ull);
         }
-        return kDone;
     };
 
     // Pairs are staged in LDS and appended to the global list by the whole workgroup: one
@@ -250,6 +280,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // bounds output-heavy joins (same-address atomics serialise at about 12 ns each).
     auto flush_stage = [&](unsigned staged) {
         const unsigned cnt = staged < (unsigned)kStagePairs ? staged : (unsigned)kStagePairs;
+        const unsigned tid = (unsigned)(wave * 64 + lane_now());
         if (tid == 0) *sFlushBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)cnt);
         __syncthreads();
         const unsigned long long gb = *sFlushBase;
@@ -260,47 +291,87 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         __syncthreads();
     };
 
-    if (tid == 0) {
-        *sStageCount = 0u;
-        *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
-    }
-    __syncthreads();
-    unsigned long long ticket = *sNext;
-
-    while (ticket != kDone) {
-        unsigned tr, tc;
-        raster_decode(p.raster, (unsigned)(ticket / p.raster.perQueue), ticket % p.raster.perQueue, &tr, &tc);
-        // padding tile of the raster, or a tile below the diagonal whose pairs its mirror tile emits
-        if (tr >= p.raster.tileRows || tc >= p.raster.tileCols || (p.symmetric && tc < tr)) {
-            __syncthreads();
-            if (tid == 0) *sNext = take(home, atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull));
-            __syncthreads();
-            ticket = *sNext;
-            continue;
-        }
-        const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
-
-        // rows past the end of the dataset re-read the last real row; their results are masked
-        const char* const gA = reinterpret_cast<const char*>(p.ptsQ + (long long)rowBase * p.ldQ16);
-        const char* const gB = reinterpret_cast<const char*>(p.ptsC + (long long)colBase * p.ldC16);
-        unsigned offA[4], offB[4];  // byte offsets from the tile's first row
+    // Byte offsets, from the tile's first row, of the 16-byte chunks this lane copies: 4 query rows and
+    // 4 candidate rows per slab.  Rows past the end of the dataset re-read the last real row; their
+    // results are masked.  The swizzle is applied here, on the global side.
+    auto tile_offsets = [&](int rowBase, int colBase, unsigned (&oA)[4], unsigned (&oB)[4]) {
+        const int ln = lane_now();
+        const int row0 = wave * 32 + (ln >> 3);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int r = cpRow0 + 8 * i;
-            const int chunk = (lane & 7) ^ swz(r);
-            offA[i] = (unsigned)(min(r, p.nQ - 1 - rowBase) * (int)p.ldQ16 + chunk) * 16u;
-            offB[i] = (unsigned)(min(r, p.nC - 1 - colBase) * (int)p.ldC16 + chunk) * 16u;
+            const int r = row0 + 8 * i;
+            const int chunk = (ln & 7) ^ swz(r);
+            oA[i] = (unsigned)(min(r, p.nQ - 1 - rowBase) * (int)p.ldQ16 + chunk) * 16u;
+            oB[i] = (unsigned)(min(r, p.nC - 1 - colBase) * (int)p.ldC16 + chunk) * 16u;
         }
-        {
-            // squared norms of the tile's 256 queries and 256 candidates, plus their maximum
-            // (it scales the safety margin of the epilogue's screening test)
-            const float mySum = tid < kTile ? p.sumsQ[min(rowBase + tid, p.nQ - 1)]
-                                            : p.sumsC[min(colBase + tid - kTile, p.nC - 1)];
-            sQ[tid] = mySum;  // sC == sQ + kTile
-            float m = __builtin_fabsf(mySum);
+    };
+
+    // One 1-KiB global->LDS transfer of this wave (global_load_lds_dwordx4: no registers in between);
+    // j = 0..7 alternates query / candidate rows.  Lane l lands in row l/8, chunk slot l%8 of the
+    // 8 rows the instruction fills; wave w owns rows [32w, 32w+32) of both operands.
+    auto issue_load = [&](const char* gA, const char* gB, const unsigned (&oA)[4], const unsigned (&oB)[4],
+                          unsigned slabByte, int stage, int j) {
+        const int i = j >> 1;
+        unsigned char* const dst = lds + stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes;
+        // uniform 64-bit base + 32-bit lane offset (formed here so it stays a 32-bit add)
+        const char* const src = (j & 1) ? gB + (oB[i] + slabByte) : gA + (oA[i] + slabByte);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    };
+
+    // Squared norms of a tile's 256 queries (waves 0-3) and 256 candidates (waves 4-7), 64 floats per
+    // wave, straight into the sums buffer `which`.
+    auto issue_sums = [&](int rowBase, int colBase, int which) {
+        const int ln = lane_now();
+        const int part = wave & 3;
+        const float* src = wave < 4 ? p.sumsQ + min(rowBase + part * 64 + ln, p.nQ - 1)
+                                    : p.sumsC + min(colBase + part * 64 + ln, p.nC - 1);
+        unsigned char* const dst = lds + kLdsSums + which * kSumsBytes + wave * 256;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
+    };
+
+    // ---- first tile
+    if (wave == 0 && lane_now() == 0) {
+        *sStageCount = 0u;
+        unsigned r, c;
+        find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r, &c);
+        sNext[0] = r;
+        sNext[1] = c;
+    }
+    __syncthreads();
+    unsigned tr = __builtin_amdgcn_readfirstlane(sNext[0]);
+    unsigned tc = __builtin_amdgcn_readfirstlane(sNext[1]);
+    if (tr == kNoTile) return;
+    __syncthreads();  // everybody has read sNext before thread 0 writes the second tile there
+
+    unsigned offA[4], offB[4];
+    tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB);
+    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)tr * kTile * p.ldQ16);
+    const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)tc * kTile * p.ldC16);
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, off, 64));
-            if (lane == 0) sWaveMax[wave] = m;
+    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0u, 0, j);
+    issue_sums((int)tr * kTile, (int)tc * kTile, 0);
+    unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
+    if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
+
+    int stage = 0;  // LDS stage that holds slab 0 of the current tile
+    int sumsBuf = 0;
+
+    for (;;) {
+        // slab 0 of this tile (issued during the previous tile's last slab) has landed
+        __syncthreads();
+        if (kEpilogue) {
+            const unsigned staged = __builtin_amdgcn_readfirstlane(*sStageCount);
+            if (staged >= (unsigned)kStagePairs / 2) flush_stage(staged);
+        }
+        if (wave == 0 && lane_now() == 0) {
+            // the reservation made a whole tile ago has long arrived: no wait here
+            unsigned r, c;
+            find_tile(popped, &r, &c);
+            sNext[0] = r;
+            sNext[1] = c;
+            popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         }
 
         floatx4 acc[kFragRows][kFragCols];
@@ -311,34 +382,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[fi][fj][r] = 0.0f;
 
-        // One 1-KiB global->LDS transfer of this wave: j = 0..7 alternates query / candidate rows.
-        auto issue_load = [&](unsigned slabByte, int stage, int j) {
-            const int i = j >> 1;
-            unsigned char* const dst = lds + stage * kStageBytes + (j & 1) * kOperandBytes +
-                                       (wave * 32 + i * 8) * kRowBytes;
-            // uniform 64-bit base + 32-bit lane offset (formed here so it stays a 32-bit add)
-            const char* const src = (j & 1) ? gB + (offB[i] + slabByte) : gA + (offA[i] + slabByte);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-        };
-#pragma unroll
-        for (int j = 0; j < 8; ++j) issue_load(0u, 0, j);
-        // reserve the next tile early so the atomic's latency hides under the k loop
-        unsigned long long nextPos = 0;
-        if (tid == 0) nextPos = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
-        __syncthreads();
-
         // One slab = 2 k-steps of 32; a k-step is two halves of 16 MFMAs (query blocks 0-3, then
         // 4-7, each against the 4 candidate blocks).  The instruction order is pinned with
         // scheduling barriers: the LDS reads for the next half are issued ahead of the MFMAs of
-        // the current half, and the 8 global->LDS transfers of the next slab are issued one per
+        // the current half, and the 8 global->LDS transfers of the following slab are issued one per
         // 4 MFMAs during the first k-step: spaced so that the texture-address queue never makes a
         // wave wait with the matrix pipe idle, early so that an L2 miss has the whole second
         // k-step to land before the slab's barrier.
-        auto slab_step = [&](int s, auto prefetch) {
-            constexpr bool kPrefetch = decltype(prefetch)::value;
-            const unsigned nextByte = (unsigned)(s + 1) * kRowBytes;
-            const unsigned char* const buf = lds + (s & 1) * kStageBytes;
+        auto slab_step = [&](int stg, bool prefetch, const char* pA, const char* pB, const unsigned (&oA)[4],
+                             const unsigned (&oB)[4], unsigned nextByte) {
+            const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[4], aHi[4], b[2][kFragCols];
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
@@ -354,7 +407,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) {
-                    if (kPrefetch && ks == 0) issue_load(nextByte, (s + 1) & 1, fj);
+                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, fj);
 #pragma unroll
                     for (int fi = 0; fi < 4; ++fi)
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
@@ -371,7 +424,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) {
-                    if (kPrefetch && ks == 0) issue_load(nextByte, (s + 1) & 1, 4 + fj);
+                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, 4 + fj);
 #pragma unroll
                     for (int fi = 0; fi < 4; ++fi)
                         acc[fi + 4][fj] =
@@ -379,13 +432,36 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            __syncthreads();
         };
-        for (int s = 0; s + 1 < p.nSlabs; ++s) slab_step(s, std::true_type{});
-        slab_step(p.nSlabs - 1, std::false_type{});
-        if (tid == 0) *sNext = take(home, nextPos);
+
+        for (int s = 0; s + 1 < p.nSlabs; ++s) {
+            slab_step(stage, true, gA, gB, offA, offB, (unsigned)(s + 1) * kRowBytes);
+            stage ^= 1;
+            __syncthreads();
+        }
+        if (p.nSlabs == 1) __syncthreads();  // with a single slab no barrier has published sNext yet
+
+        // The tile after this one: its first slab and its squared norms travel during this tile's last
+        // slab and epilogue.  The current tile's offsets are not needed any more, so the next tile's
+        // take their registers.
+        const unsigned ntr = __builtin_amdgcn_readfirstlane(sNext[0]);
+        const unsigned ntc = __builtin_amdgcn_readfirstlane(sNext[1]);
+        const bool more = ntr != kNoTile;
+        if (more) {
+            tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB);
+            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
+            gB = reinterpret_cast<const char*>(p.ptsC + (long long)ntc * kTile * p.ldC16);
+            issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
+        }
+        slab_step(stage, more, gA, gB, offA, offB, 0u);
+        stage ^= 1;
 
         if (kEpilogue) {
+            const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
+            const int ln = lane_now();
+            const int l16 = ln & 15, quad = ln >> 4;
+            const float* const sQ = reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes);
+            const float* const sC = sQ + kTile;
             const int qBase = rowBase + wr * kWaveRows;
             int cand[kFragCols];
             float sc[kFragCols];
@@ -395,11 +471,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
             }
             // margin of the screening test: covers the FP32 roundings of both forms of the inequality
-            const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
-            float sMax = sWaveMax[0];
+            // for every element of this wave's block (largest squared norm among its rows and columns)
+            float sMax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(sQ[wr * kWaveRows + ln]),
+                                                         __builtin_fabsf(sQ[wr * kWaveRows + 64 + ln])),
+                                         __builtin_fabsf(sC[wc * kWaveCols + ln]));
 #pragma unroll
-            for (int w = 1; w < 8; ++w) sMax = __builtin_fmaxf(sMax, sWaveMax[w]);
+            for (int off = 32; off > 0; off >>= 1)
+                sMax = __builtin_fmaxf(sMax, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(
+                                                 (ln ^ off) << 2, __builtin_bit_cast(int, sMax))));
             const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
+            const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
             unsigned mask[kFragRows / 2];
             if (edge)
                 test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
@@ -419,35 +500,46 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 int incl = mine;
 #pragma unroll
                 for (int off = 1; off < 64; off <<= 1) {
-                    const int v = __shfl_up(incl, off, 64);
-                    if (lane >= off) incl += v;
+                    const int v = __builtin_amdgcn_ds_bpermute((ln - off) << 2, incl);
+                    if (ln >= off) incl += v;
                 }
-                const unsigned total = (unsigned)__shfl(incl, 63, 64);
+                const unsigned total = (unsigned)__builtin_amdgcn_readlane(incl, 63);
                 // reserve room in the staging area (LDS atomic); what does not fit goes straight
                 // to the global list with a reservation of this wave's own
+                // (LDS atomic and LDS stores below are written as instructions: for ordinary LDS writes the
+                // compiler first waits until this wave's global->LDS transfers of the next tile have landed)
                 unsigned pos = 0;
-                if (lane == 0) pos = atomicAdd(sStageCount, total);
-                pos = __shfl(pos, 0, 64);
+                if (ln == 0)
+                    asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=v"(pos)
+                                 : "v"(ldsBase + (unsigned)kLdsStageCount), "v"(total)
+                                 : "memory");
+                pos = __builtin_amdgcn_readfirstlane(pos);
                 const unsigned room = pos < (unsigned)kStagePairs ? (unsigned)kStagePairs - pos : 0u;
                 const unsigned fit = total < room ? total : room;
                 unsigned long long gbase = 0;
                 if (fit < total) {
-                    if (lane == 0) gbase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)(total - fit));
-                    gbase = __shfl(gbase, 0, 64);
+                    if (ln == 0) gbase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)(total - fit));
+                    gbase = ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(gbase >> 32)) << 32) |
+                            __builtin_amdgcn_readfirstlane((unsigned)gbase);
                 }
                 unsigned idx = (unsigned)(incl - mine);
 #pragma unroll
                 for (int fp = 0; fp < kFragRows / 2; ++fp) {
                     unsigned m = mask[fp];
                     while (m) {
-                        const int bit = __builtin_ctz(m);
+                        const int low = __builtin_ctz(m);
                         m &= m - 1;
+                        const int bit = 31 - low;  // element number inside the pair of row blocks
                         const int fi = fp * 2 + (bit >> 4), fj = (bit >> 2) & 3, r = bit & 3;
                         const int q = qBase + fi * 16 + quad * 4 + r;
                         const int c = colBase + wc * kWaveCols + fj * 16 + l16;
                         auto put = [&](unsigned at, int first, int second) {
                             if (at < fit) {
-                                sStage[pos + at] = make_int2(first, second);
+                                const unsigned long long rec =
+                                    (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
+                                asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage + (pos + at) * 8u), "v"(rec)
+                                             : "memory");
                             } else {
                                 const unsigned long long slot = gbase + (at - fit);
                                 if (slot < p.cap) p.pairs[slot] = make_int2(first, second);
@@ -457,6 +549,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         if (mirror) put(idx++, c, q);
                     }
                 }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staged records are in LDS
             }
         } else {
             // keep the accumulators observable without spending instructions on them
@@ -465,15 +558,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int fj = 0; fj < kFragCols; ++fj) asm volatile("" ::"v"(acc[fi][fj]));
         }
-        __syncthreads();
-        ticket = *sNext;
-        if (kEpilogue) {
-            const unsigned staged = *sStageCount;  // uniform: read after the barrier
-            if (staged >= (unsigned)kStagePairs / 2) flush_stage(staged);
-        }
+
+        if (!more) break;
+        tr = ntr;
+        tc = ntc;
+        sumsBuf ^= 1;
     }
     if (kEpilogue) {
-        const unsigned staged = *sStageCount;
+        __syncthreads();
+        const unsigned staged = __builtin_amdgcn_readfirstlane(*sStageCount);
         if (staged > 0) flush_stage(staged);
     }
 }
@@ -532,12 +625,6 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
         e = hipGetDeviceProperties(&prop, dev);
         if (e != hipSuccess) return e;
         numCUs = prop.multiProcessorCount;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&join_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&join_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return e;
         configured = true;
     }
     JoinParams p;
@@ -561,9 +648,9 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
     unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
     if (l.epilogue)
-        join_kernel<true><<<dim3(grid), dim3(kThreads), kLdsBytes, stream>>>(p);
+        join_kernel<true><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
     else
-        join_kernel<false><<<dim3(grid), dim3(kThreads), kLdsBytes, stream>>>(p);
+        join_kernel<false><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
     return hipGetLastError();
 }
 
