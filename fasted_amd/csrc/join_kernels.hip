@@ -151,46 +151,56 @@ struct JoinParams {
 // Distance test of one wave's 128x64 block of accumulators.  acc[fi][fj] is a 16x16 MFMA block:
 // lane l holds column l%16 and rows 4*(l/16) .. +3, i.e. 4 elements per block.
 //
-// Screening, 1.75 VALU ops per element: in real arithmetic a hit is
-//     acc - s_q/2 >= (s_c - eps^2)/2,
-// so per block the maximum of acc - s_q/2 over the lane's 4 rows is compared with the column's
-// right-hand side minus `margin`, which covers every FP32 rounding of both forms.  The compare is
-// wave-wide (its result is the ballot), and only blocks in which some lane has a candidate evaluate
-// the reference formula exactly:  (s_q + s_c) - 2*acc <= eps^2  in FP32 (source/warpMma.cuh:241-257).
+// The accumulators start at -(s_q + s_c)/2 instead of 0, so what arrives here is
+//     a = q.c - (s_q + s_c)/2 = -dist^2 / 2
+// and the reference's test  s_q + s_c - 2 q.c <= eps^2  (source/warpMma.cuh:241-257) reads
+//     a >= -eps^2/2,
+// one threshold for every element, exact in FP32 (the scaling by 2 is exact), and symmetric in q and c
+// like the reference's.  Screening, 1/3 VALU op per element: the maximum of the lane's 128 elements
+// against the threshold; a wave in which no lane has a hit is done.  Otherwise the blocks are screened
+// one by one (maximum of the lane's 4 rows, wave-wide ballot) and the blocks with a hit yield their
+// per-element bits.
 //
-// kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; every block is
-// evaluated exactly, self pairs are forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
+// kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; self pairs are
+// forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
 // Returns per-lane hit bits, shifted in from the right in evaluation order: element e = (fi&1)*16 + fj*4 + r
 // of the pair of row blocks fi/2 ends up in bit 31 - e of mask[fi/2].
 template <bool kEdge>
-__device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const float* sQ,
-                                           const float (&sc)[kFragCols], const int (&cand)[kFragCols], int qBase,
-                                           int quad, int nQ, int nC, int selfJoin, float eps2, float margin,
+__device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const int (&cand)[kFragCols],
+                                           int qBase, int quad, int nQ, int nC, int selfJoin, float thr,
                                            unsigned (&mask)[kFragRows / 2]) {
-    float thr[kFragCols];
+    if (!kEdge) {
+        float best = acc[0][0][0];
 #pragma unroll
-    for (int fj = 0; fj < kFragCols; ++fj) thr[fj] = 0.5f * (sc[fj] - eps2) - margin;
+        for (int fi = 0; fi < kFragRows; ++fi)
+#pragma unroll
+            for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) best = __builtin_fmaxf(best, acc[fi][fj][r]);
+        if (__builtin_amdgcn_ballot_w64(best >= thr) == 0ull) {
+#pragma unroll
+            for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
+            return;
+        }
+    }
 #pragma unroll
     for (int fp = 0; fp < kFragRows / 2; ++fp) {
         unsigned m = 0;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int fi = fp * 2 + h;
-            const floatx4 sq = *reinterpret_cast<const floatx4*>(sQ + fi * 16 + quad * 4);
-            const floatx4 hq = sq * 0.5f;
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj) {
                 bool look = kEdge;
                 if (!kEdge) {
-                    const floatx4 f = acc[fi][fj] - hq;
+                    const floatx4 f = acc[fi][fj];
                     const float best = __builtin_fmaxf(__builtin_fmaxf(f[0], f[1]), __builtin_fmaxf(f[2], f[3]));
-                    look = __builtin_amdgcn_ballot_w64(best >= thr[fj]) != 0ull;
+                    look = __builtin_amdgcn_ballot_w64(best >= thr) != 0ull;
                 }
                 if (look) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const float d2 = (sq[r] + sc[fj]) - (2.0f * acc[fi][fj][r]);
-                        bool hit = d2 <= eps2;
+                        bool hit = acc[fi][fj][r] >= thr;
                         if (kEdge) {
                             const int q = qBase + fi * 16 + quad * 4 + r;
                             hit = (hit || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
@@ -374,13 +384,25 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         }
 
+        // the accumulators start at -(s_q + s_c)/2 (see test_block): the tile's squared norms landed
+        // together with slab 0
         floatx4 acc[kFragRows][kFragCols];
+        {
+            const int ln = lane_now();
+            const float* const sQw =
+                reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + wr * kWaveRows + (ln >> 4) * 4;
+            const float* const sCw =
+                reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + kTile + wc * kWaveCols + (ln & 15);
+            float hc[kFragCols];
 #pragma unroll
-        for (int fi = 0; fi < kFragRows; ++fi)
+            for (int fj = 0; fj < kFragCols; ++fj) hc[fj] = -0.5f * sCw[fj * 16];
 #pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj)
+            for (int fi = 0; fi < kFragRows; ++fi) {
+                const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16) * -0.5f;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[fi][fj][r] = 0.0f;
+                for (int fj = 0; fj < kFragCols; ++fj) acc[fi][fj] = hq + hc[fj];
+            }
+        }
 
         // One slab = 2 k-steps of 32; a k-step is two halves of 16 MFMAs (query blocks 0-3, then
         // 4-7, each against the 4 candidate blocks).  The instruction order is pinned with
@@ -460,34 +482,17 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
             const int ln = lane_now();
             const int l16 = ln & 15, quad = ln >> 4;
-            const float* const sQ = reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes);
-            const float* const sC = sQ + kTile;
             const int qBase = rowBase + wr * kWaveRows;
             int cand[kFragCols];
-            float sc[kFragCols];
 #pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj) {
-                cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
-                sc[fj] = sC[wc * kWaveCols + fj * 16 + l16];
-            }
-            // margin of the screening test: covers the FP32 roundings of both forms of the inequality
-            // for every element of this wave's block (largest squared norm among its rows and columns)
-            float sMax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(sQ[wr * kWaveRows + ln]),
-                                                         __builtin_fabsf(sQ[wr * kWaveRows + 64 + ln])),
-                                         __builtin_fabsf(sC[wc * kWaveCols + ln]));
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1)
-                sMax = __builtin_fmaxf(sMax, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(
-                                                 (ln ^ off) << 2, __builtin_bit_cast(int, sMax))));
-            const float margin = (2.0f * sMax + __builtin_fabsf(p.eps2)) * 0x1p-18f;
+            for (int fj = 0; fj < kFragCols; ++fj) cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
+            const float thr = -0.5f * p.eps2;
             const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
             unsigned mask[kFragRows / 2];
             if (edge)
-                test_block<true>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
-                                 mask);
+                test_block<true>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
             else
-                test_block<false>(acc, sQ + wr * kWaveRows, sc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, p.eps2, margin,
-                                  mask);
+                test_block<false>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
 
             // symmetric mode: a tile above the diagonal also stands for its mirror image
             const bool mirror = p.symmetric && tr != tc;
