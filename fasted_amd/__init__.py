@@ -19,11 +19,12 @@ from .find_pairs import (  # noqa: F401
     mmaShape,
     resident_points,
     self_join,
+    self_join_blocked,
     self_join_device,
     sum_squared_device,
 )
 
 __all__ = [
     "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "join_device", "library_path",
-    "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_device", "sum_squared_device",
+    "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_blocked", "self_join_device", "sum_squared_device",
 ]

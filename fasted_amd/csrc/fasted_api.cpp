@@ -7,6 +7,7 @@
 // that reRun() can change epsilon without touching the data (source/main.cu:33,198-248).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cmath>
 #include <climits>
@@ -151,7 +152,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.pairs = dPairs;
     jl.cap = cap;
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
-    HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, stream));
+    HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, stream));
     HIP_CHECK(fasted::launch_join(jl, stream));
     HIP_CHECK(hipEventRecord(t.ev[2], stream));
     HIP_CHECK(hipStreamSynchronize(stream));
@@ -178,6 +179,142 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
         stats->pairsFound = cnt[0];
         stats->pairsStored = cnt[1];
     }
+}
+
+// Self-join of a host-resident dataset that is streamed through the device in blocks of `blockRows`
+// points: for every query block (held on the device) every candidate block is uploaded in turn, on a
+// copy stream, while the join of the block before it runs.  The pairs of one query block are appended
+// to one device buffer across the candidate blocks, get their global indices, are sorted row-major and
+// go back to the host; query blocks are processed in order, so the whole output is row-major.
+struct DeviceBuffers {
+    std::vector<void*> owned;
+    hipStream_t compute = nullptr, copy = nullptr;
+    ~DeviceBuffers() {
+        for (void* p : owned) (void)hipFree(p);
+        if (compute) (void)hipStreamDestroy(compute);
+        if (copy) (void)hipStreamDestroy(copy);
+    }
+    void* alloc(size_t bytes) {
+        void* p = nullptr;
+        HIP_CHECK(hipMalloc(&p, bytes ? bytes : 1));
+        owned.push_back(p);
+        return p;
+    }
+};
+
+void self_join_blocked(const uint16_t* points, long long n, int d, double epsilon, long long blockRows, FastedPair* out,
+                       unsigned long long cap, unsigned long long* found, unsigned long long* stored) {
+    if (!points) throw std::invalid_argument("points pointer is null");
+    if (cap > 0 && !out) throw std::invalid_argument("output buffer is null");
+    if (blockRows < 1) throw std::invalid_argument("block size must be at least 1 point");
+    const int dPad = round_up(d, fasted::kSlabK);
+    validate_shape(n, d, dPad);
+    // blocks start on tile boundaries, so a block join sees the same tiles as the whole join would
+    const long long rows = std::min<long long>(round_up(blockRows, fasted::kTile), round_up(n, fasted::kTile));
+    const long long blocks = (n + rows - 1) / rows;
+    const size_t pitch = (size_t)dPad * 2, blockBytes = (size_t)rows * pitch;
+
+    DeviceBuffers dev;
+    HIP_CHECK(hipStreamCreateWithFlags(&dev.compute, hipStreamNonBlocking));
+    HIP_CHECK(hipStreamCreateWithFlags(&dev.copy, hipStreamNonBlocking));
+    void* qBlock = dev.alloc(blockBytes);
+    void* cBlock[2] = {dev.alloc(blockBytes), dev.alloc(blockBytes)};
+    float* qSums = static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)));
+    float* cSums[2] = {static_cast<float*>(dev.alloc((size_t)rows * sizeof(float))),
+                       static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)))};
+    if (dPad != d) {  // the columns d..dPad are never written again and must read as zeros
+        HIP_CHECK(hipMemset(qBlock, 0, blockBytes));
+        HIP_CHECK(hipMemset(cBlock[0], 0, blockBytes));
+        HIP_CHECK(hipMemset(cBlock[1], 0, blockBytes));
+    }
+    // pair buffer of one query block: rows*256 records as the reference sizes its buffer per point
+    // (source/findPairs.cuh:644-647), shrunk to half of what is free (the sort needs as much again)
+    unsigned long long devCap = std::min<unsigned long long>((unsigned long long)rows * 256ull, cap);
+    size_t freeB = 0, totalB = 0;
+    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
+    devCap = std::min<unsigned long long>(devCap, (unsigned long long)(freeB / 2) / sizeof(FastedPair));
+    void* dPairs = dev.alloc((size_t)devCap * sizeof(FastedPair));
+    g_ws.ensure(1);
+
+    auto block_rows = [&](long long b) { return std::min<long long>(rows, n - b * rows); };
+    auto upload = [&](void* dst, long long b, hipStream_t s) {
+        HIP_CHECK(hipMemcpy2DAsync(dst, pitch, points + (size_t)b * rows * d, (size_t)d * 2, (size_t)d * 2,
+                                   (size_t)block_rows(b), hipMemcpyHostToDevice, s));
+    };
+    unsigned long long foundAll = 0, storedAll = 0;
+    const float eps2 = static_cast<float>(epsilon * epsilon);
+    for (long long i = 0; i < blocks; ++i) {
+        const int nQ = (int)block_rows(i);
+        upload(qBlock, i, dev.compute);
+        HIP_CHECK(fasted::launch_sum_squared(qBlock, dPad, nQ, dPad, qSums, dev.compute));
+        HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, dev.compute));
+        unsigned long long before = 0;  // pairs of this query block found so far
+        // candidate blocks other than block i itself pass through the two buffers in turn; `nextUp` is the
+        // block to upload next, cBlock[slot] the buffer the next such join reads
+        auto other_after = [&](long long b) { return (b + 1 == i) ? b + 2 : b + 1; };
+        long long nextUp = (i == 0) ? 1 : 0;
+        int slot = 0;
+        if (nextUp < blocks) {
+            upload(cBlock[0], nextUp, dev.copy);
+            nextUp = other_after(nextUp);
+        }
+        for (long long j = 0; j < blocks; ++j) {
+            const bool diagonal = (j == i);
+            const void* cand = qBlock;
+            const float* candSums = qSums;
+            int nC = nQ;
+            if (!diagonal) {
+                HIP_CHECK(hipStreamSynchronize(dev.copy));  // block j has arrived in cBlock[slot]
+                cand = cBlock[slot];
+                candSums = cSums[slot];
+                nC = (int)block_rows(j);
+                HIP_CHECK(fasted::launch_sum_squared(cand, dPad, nC, dPad, cSums[slot], dev.compute));
+            }
+            fasted::JoinLaunch jl;
+            jl.queries = qBlock;
+            jl.candidates = cand;
+            jl.ldQ = jl.ldC = dPad;
+            jl.nQ = nQ;
+            jl.nC = nC;
+            jl.selfJoin = diagonal;
+            jl.symmetric = false;
+            jl.dPad = dPad;
+            jl.eps2 = eps2;
+            jl.sumsQ = qSums;
+            jl.sumsC = candSums;
+            jl.counters = g_ws.counters;
+            jl.pairs = dPairs;
+            jl.cap = devCap;
+            jl.epilogue = true;
+            HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, /*keepFound=*/true, dev.compute));
+            HIP_CHECK(fasted::launch_join(jl, dev.compute));
+            if (!diagonal) {
+                // the next candidate block travels while this join runs; the other buffer was last read
+                // by a join that has finished (its counter was read back)
+                slot ^= 1;
+                if (nextUp < blocks) {
+                    upload(cBlock[slot], nextUp, dev.copy);
+                    nextUp = other_after(nextUp);
+                }
+            }
+            HIP_CHECK(hipStreamSynchronize(dev.compute));
+            unsigned long long after = 0;
+            HIP_CHECK(hipMemcpy(&after, g_ws.counters, sizeof after, hipMemcpyDeviceToHost));
+            HIP_CHECK(fasted::launch_offset_pairs(dPairs, std::min(before, devCap), std::min(after, devCap),
+                                                  (int)(i * rows), (int)(j * rows), dev.compute));
+            before = after;
+        }
+        const unsigned long long kept = std::min(before, devCap);
+        if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute));
+        HIP_CHECK(hipStreamSynchronize(dev.compute));
+        const unsigned long long take = std::min(kept, cap - storedAll);
+        if (take)
+            HIP_CHECK(hipMemcpy(out + storedAll, dPairs, (size_t)take * sizeof(FastedPair), hipMemcpyDeviceToHost));
+        storedAll += take;
+        foundAll += before;
+    }
+    if (found) *found = foundAll;
+    if (stored) *stored = storedAll;
 }
 
 // ---- resident dataset of the reference-compatible entry points -------------------------
@@ -461,6 +598,12 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
         (void)hipFree(dPoints);
         (void)hipFree(dPairs);
     });
+}
+
+int fasted_self_join_blocked(const uint16_t* points, long long n, int d, double epsilon, long long block_rows,
+                             FastedPair* out, unsigned long long cap, unsigned long long* found,
+                             unsigned long long* stored) {
+    return guarded([&] { self_join_blocked(points, n, d, epsilon, block_rows, out, cap, found, stored); });
 }
 
 int fasted_load_exponential_dataset(int size, int dimensionality, double lambda, double max) {

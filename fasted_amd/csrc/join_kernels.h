@@ -36,7 +36,11 @@ unsigned long long tile_count(long long nQ, long long nC);  // 256x256 tiles the
 int lds_chunk_slot(int row, int chunk);
 
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream);
-hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream);
+// Clears the queue heads and, unless keepFound, the pair counter (word 0 of `counters`).
+hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream);
+// pairs[first, last): QueryPoint += qOffset, CandidatePoint += cOffset.
+hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,
+                               hipStream_t stream);
 hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
 
 // Row-major sort of `count` stored pairs (pair_sort.hip).

@@ -126,8 +126,23 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
     if (sub == 0 && row < n) sums[row] = acc;
 }
 
-__global__ void reset_counters_kernel(unsigned long long* c) {
-    if (threadIdx.x < kCounterWords) c[threadIdx.x] = 0ull;
+// Clears the queue heads and, unless `keepFound`, the pair counter (word 0): a launch that keeps it
+// appends its pairs behind those of the launch before.
+__global__ void reset_counters_kernel(unsigned long long* c, int keepFound) {
+    if (threadIdx.x < kCounterWords && !(keepFound && threadIdx.x == kCounterFound)) c[threadIdx.x] = 0ull;
+}
+
+// Adds the first row of the query block and of the candidate block to the pairs [first, last) that a
+// join of two row blocks of a larger dataset has appended with block-local indices.
+__global__ void __launch_bounds__(256) offset_pairs_kernel(int2* pairs, unsigned long long first,
+                                                           unsigned long long last, int qOffset, int cOffset) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = first + (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < last; i += stride) {
+        int2 v = pairs[i];
+        v.x += qOffset;
+        v.y += cOffset;
+        pairs[i] = v;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -614,8 +629,17 @@ hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad,
     return hipGetLastError();
 }
 
-hipError_t launch_reset_counters(unsigned long long* counters, hipStream_t stream) {
-    reset_counters_kernel<<<1, 256, 0, stream>>>(counters);
+hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream) {
+    reset_counters_kernel<<<1, 256, 0, stream>>>(counters, keepFound ? 1 : 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,
+                               hipStream_t stream) {
+    if (last <= first || (qOffset == 0 && cOffset == 0)) return hipSuccess;
+    const unsigned long long count = last - first;
+    const unsigned blocks = (unsigned)((count + 255) / 256 < 4096 ? (count + 255) / 256 : 4096);
+    offset_pairs_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(static_cast<int2*>(pairs), first, last, qOffset, cOffset);
     return hipGetLastError();
 }
 

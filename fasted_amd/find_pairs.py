@@ -109,6 +109,9 @@ def load_findpairs(path: str = None):
     lib.fasted_self_join.restype = c.c_int
     lib.fasted_self_join.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_double, c.c_void_p, c.c_ulonglong,
                                      c.POINTER(c.c_ulonglong), c.POINTER(c.c_ulonglong)]
+    lib.fasted_self_join_blocked.restype = c.c_int
+    lib.fasted_self_join_blocked.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_double, c.c_longlong, c.c_void_p,
+                                             c.c_ulonglong, c.POINTER(c.c_ulonglong), c.POINTER(c.c_ulonglong)]
     lib.fasted_self_join_device.restype = c.c_int
     lib.fasted_self_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_double, c.c_void_p,
                                             c.c_void_p, c.c_ulonglong, c.c_uint, c.c_void_p,
@@ -169,6 +172,25 @@ def self_join(points_fp16, epsilon, cap=None):
     found, stored = ctypes.c_ulonglong(), ctypes.c_ulonglong()
     _check(lib, lib.fasted_self_join(a.ctypes.data, n, d, float(epsilon), out.ctypes.data, cap,
                                      ctypes.byref(found), ctypes.byref(stored)))
+    return out[:stored.value], found.value
+
+
+def self_join_blocked(points_fp16, epsilon, block_rows, cap=None):
+    """self_join for a dataset streamed through the device in blocks of `block_rows` points."""
+    import numpy as np
+
+    lib = load_findpairs()
+    a = np.ascontiguousarray(points_fp16)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    if a.dtype != np.uint16 or a.ndim != 2:
+        raise TypeError("points must be a 2-D float16 / uint16 array")
+    n, d = a.shape
+    cap = int(cap if cap is not None else n * 256)
+    out = np.empty((max(cap, 1), 2), dtype=np.int32)
+    found, stored = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+    _check(lib, lib.fasted_self_join_blocked(a.ctypes.data, n, d, float(epsilon), int(block_rows), out.ctypes.data, cap,
+                                             ctypes.byref(found), ctypes.byref(stored)))
     return out[:stored.value], found.value
 
 

@@ -98,6 +98,18 @@ enum {
 int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon, FastedPair* out,
                      unsigned long long cap, unsigned long long* found, unsigned long long* stored);
 
+/* The same join for a dataset that does not fit the device (or should not occupy it): the host-resident
+ * points are streamed through the device in blocks of `block_rows` points (rounded up to a multiple of
+ * 256).  Device memory used: three blocks, their norms, and a pair buffer of min(cap, block_rows*256)
+ * records (twice that while sorting).  Output as fasted_self_join: row-major, *found counts every pair,
+ * at most `cap` are written; in addition the pairs of one block of query points beyond block_rows*256 are
+ * counted but not written.  The reference has no such path: its dataset, twice, and N*256 pair records
+ * must fit the device (source/findPairs.cuh:568-600,644-647); "batching" is named as future work in its
+ * paper. */
+int fasted_self_join_blocked(const uint16_t* points, long long n, int d, double epsilon, long long block_rows,
+                             FastedPair* out, unsigned long long cap, unsigned long long* found,
+                             unsigned long long* stored);
+
 /* Everything already in device memory (HBM-resident dataset, caller-owned pair buffer).
  *   d_points   N rows of FP16, row stride `ld` halves (ld % 8 == 0, ld >= D rounded up to
  *              64; the columns D..roundup(D,64) of every row must be readable zeros, or

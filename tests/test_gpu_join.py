@@ -236,3 +236,27 @@ def test_symmetric_option_gives_the_same_pair_set(fasted, n, d):
     assert st_half.pairsFound == st_full.pairsFound
     assert np.array_equal(half, full)
     check_against_fp64(bits, n, eps, half)
+
+
+@pytest.mark.parametrize("n,d,block", [(3000, 100, 1024), (2600, 64, 256), (1500, 192, 4096), (5000, 128, 1000)])
+def test_blocked_join_equals_the_whole_join(fasted, n, d, block):
+    """The dataset streamed through the device in row blocks gives the pair list of the one-shot join,
+    record for record (same arithmetic per pair, row-major order across the blocks)."""
+    bits = datasets.uniform_bytes(n, d, seed=11 * n + d)
+    eps = datasets.epsilon_for_neighbours(bits, 15)
+    whole, found_whole = fasted.self_join(bits, eps)
+    blocked, found_blocked = fasted.self_join_blocked(bits, eps, block)
+    assert found_blocked == found_whole == len(whole)
+    assert np.array_equal(blocked, whole)
+    check_against_fp64(bits, n, eps, blocked)
+
+
+def test_blocked_join_overflow_is_soft(fasted):
+    n, d = 2000, 64
+    bits = datasets.uniform_bytes(n, d, seed=21)
+    eps = datasets.epsilon_for_neighbours(bits, 20)
+    whole, found_whole = fasted.self_join(bits, eps)
+    cap = len(whole) // 3
+    part, found = fasted.self_join_blocked(bits, eps, 512, cap=cap)
+    assert found == found_whole and len(part) == cap
+    assert np.array_equal(part, whole[:cap])  # row-major prefix: the first query blocks come first
