@@ -304,3 +304,100 @@ def test_host_quantisation_rounds_twice_like_the_reference(lib, tmp_path):
     assert (n, d) == (len(tricky), 1)
     assert np.array_equal(bits[:n, 0], tricky.astype(np.float32).astype(np.float16).view(np.uint16))
     assert np.array_equal(bits[:n, 0], oracle.quantize(tricky))
+
+
+# ---------------------------------------------------------------- experiment driver
+class MockBackend:
+    """Backend in the manner of the reference's MockFindPairs (results/scripts/tests/
+    test_experiments.py:14-71): the selectivity equals epsilon, nothing is computed."""
+
+    def __init__(self):
+        self.size, self.dim, self.log = 0, 0, []
+
+    def _result(self, epsilon):
+        r = fp.Results()
+        r.TFLOPS = 1.0
+        r.pairsFound = r.pairsStored = int(epsilon * self.size) + self.size
+        r.inputProblemShape = fp.mmaShape(self.size, self.size, self.dim)
+        r.paddedProblemShape = fp.mmaShape(self.size, self.size, self.dim)
+        return r
+
+    def runFromExponentialDataset(self, size, dim, e_lambda, e_range, epsilon, save_pairs):
+        self.size, self.dim = size, dim
+        self.log.append(("exp", size, dim, e_lambda, e_range, epsilon, save_pairs))
+        return self._result(epsilon)
+
+    def runFromFile(self, filename, epsilon, save_pairs):
+        self.size, self.dim = 100000, 15
+        self.log.append(("file", filename, epsilon, save_pairs))
+        return self._result(epsilon)
+
+    def reRun(self, epsilon, save_pairs):
+        self.log.append(("rerun", epsilon, save_pairs))
+        return self._result(epsilon)
+
+
+def reference_record_keys():
+    with open(os.path.join(os.path.dirname(__file__), "golden", "speed_results_records.json")) as f:
+        gold = json.load(f)
+    rec = gold["sweep"][0]
+    return set(rec), set(rec["results"]), gold
+
+
+def test_experiment_runner_writes_the_reference_result_schema(tmp_path):
+    from fasted_amd import experiments as ex
+
+    top, inner, _ = reference_record_keys()
+    backend = MockBackend()
+    runner = ex.ExperimentRunner(backend, output_dir=str(tmp_path))
+
+    # size x dimensionality sweep: 3 timed runs per shape, dataset built once per shape
+    path = runner.run_speed_sweeps_exponential_data_experiment(sizes=[1000, 2154], dims=[64, 128])
+    records = json.load(open(path))
+    assert len(records) == 2 * 2 * 3
+    for r in records:
+        assert set(r) == top and inner <= set(r["results"])
+        assert r["epsilon"] == 0.001 and r["selectivity"] == 0
+        assert r["results"]["inputProblemShape"]["m"] in (1000, 2154)
+    assert [r["iteration"] for r in records[:3]] == [0, 1, 2]
+    builds = [e for e in backend.log if e[0] == "exp"]
+    assert [(e[1], e[2]) for e in builds] == [(1000, 64), (1000, 128), (2154, 64), (2154, 128)]
+    assert all(e[3:5] == (40, 10) for e in builds)  # lambda 40, range 10 (experiments.py:556-557)
+    assert len([e for e in backend.log if e[0] == "rerun"]) == 8
+
+    # selectivity experiment: epsilon found per target (selectivity == epsilon for the mock), 3 runs each
+    backend.log.clear()
+    path = runner.run_selectivity_vs_speed_experiment([1, 10, 100], size=5000, dim=64)
+    records = json.load(open(path))
+    assert len(records) == 9 and [r["selectivity"] for r in records[::3]] == [1, 10, 100]
+    for r in records:
+        assert ex.within_percent(r["epsilon"], r["selectivity"], 0.011)
+    assert len([e for e in backend.log if e[0] == "exp"]) == 1  # one build, everything else reRun
+
+    # known epsilons on a file: rebuilt for every run, pairs saved on the first run of a parameter set only
+    backend.log.clear()
+    params = [ex.SearchParameters(64, 1.2, True), ex.SearchParameters(128, 3.4, False)]
+    path = runner.run_real_dataset_known_epsilons_experiments("base", "data.csv", params, num_repetitions=2)
+    assert os.path.basename(path).startswith("data.csv_results_")
+    assert [e[1:] for e in backend.log] == [(b"base/data.csv", 1.2, True), (b"base/data.csv", 1.2, False),
+                                            (b"base/data.csv", 3.4, False), (b"base/data.csv", 3.4, False)]
+
+    # epsilon finder over datasets: a dictionary of record lists keyed by dataset
+    path = runner.run_real_datasets_epsilon_finder_experiments([1, 10], base_path="base", datasets=["a.txt", "b.txt"])
+    by_dataset = json.load(open(path))
+    assert set(by_dataset) == {"a.txt", "b.txt"} and all(len(v) == 2 for v in by_dataset.values())
+
+
+def test_time_trials_skip_failed_runs():
+    from fasted_amd import experiments as ex
+
+    calls = []
+
+    def finder(eps, save):
+        calls.append((eps, save))
+        if len(calls) == 2:
+            raise RuntimeError("device lost")
+        return fp.Results()
+
+    out = ex.ExperimentRunner(None).run_time_trials(finder, [ex.SearchParameters(1, 0.5, True)], 3)
+    assert [e.iteration for e in out] == [0, 2] and calls == [(0.5, True), (0.5, False), (0.5, False)]

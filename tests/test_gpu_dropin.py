@@ -113,3 +113,31 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     truth = oracle.self_join_f64(bits, eps, n=n)
     assert abs(int(found) - len(truth)) <= max(4, len(truth) // 500)
     lib.releaseResources()
+
+
+def test_experiment_sweep_reproduces_the_reference_result_records(lib, tmp_path):
+    """The size x dimensionality sweep of the reference's experiment driver, run on the library: for
+    the shapes small enough to run here the records of results/speed_results/
+    ExpoDataSpeedVsSize_OnDemandRasterizer.json (pairs found, input shape, epsilon) are reproduced."""
+    import json
+
+    from fasted_amd import experiments as ex
+
+    with open(os.path.join(ROOT, "tests", "golden", "speed_results_records.json")) as f:
+        gold = json.load(f)["sweep"]
+    sizes = sorted({r["results"]["inputProblemShape"]["m"] for r in gold})
+    dims = sorted({r["results"]["inputProblemShape"]["k"] for r in gold})
+    runner = ex.ExperimentRunner(lib, output_dir=str(tmp_path))
+    records = json.load(open(runner.run_speed_sweeps_exponential_data_experiment(sizes=sizes, dims=dims, iterations=1)))
+    key = lambda r: (r["results"]["inputProblemShape"]["m"], r["results"]["inputProblemShape"]["k"])
+    ours = {key(r): r for r in records}
+    assert len(ours) == len(gold)
+    for g in gold:
+        r = ours[key(g)]
+        assert set(g) == set(r) and set(g["results"]) <= set(r["results"])
+        assert (r["selectivity"], r["epsilon"], r["iteration"]) == (g["selectivity"], g["epsilon"], g["iteration"])
+        for field in ("pairsFound", "pairsStored", "inputProblemShape"):
+            assert r["results"][field] == g["results"][field], (field, key(g))
+        assert r["results"]["paddedProblemShape"]["k"] == g["results"]["paddedProblemShape"]["k"]
+        assert r["results"]["TFLOPS"] > 0
+    lib.releaseResources()
