@@ -17,6 +17,7 @@ from .find_pairs import (  # noqa: F401
     library_path,
     load_findpairs,
     mmaShape,
+    pair_distances_device,
     resident_points,
     self_join,
     self_join_blocked,
@@ -26,5 +27,5 @@ from .find_pairs import (  # noqa: F401
 
 __all__ = [
     "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "join_device", "library_path",
-    "load_findpairs", "mmaShape", "resident_points", "self_join", "self_join_blocked", "self_join_device", "sum_squared_device",
+    "load_findpairs", "mmaShape", "pair_distances_device", "resident_points", "self_join", "self_join_blocked", "self_join_device", "sum_squared_device",
 ]

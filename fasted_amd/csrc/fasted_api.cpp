@@ -335,11 +335,24 @@ std::string output_dir() {
     return env && *env ? std::string(env) : std::string(".");
 }
 
-void write_pairs_text(const std::string& path, const std::vector<FastedPair>& pairs) {
+bool g_saveDistances = false;
+
+bool save_distances() {
+    if (g_saveDistances) return true;
+    const char* v = std::getenv("FASTED_PAIRS_DISTANCES");
+    return v && *v && *v != '0';
+}
+
+void write_pairs_text(const std::string& path, const std::vector<FastedPair>& pairs, const std::vector<float>& dist) {
     std::FILE* f = std::fopen(path.c_str(), "w");
     if (!f) throw std::ios_base::failure("Failed to open output file: " + path);
-    // "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54
-    for (const FastedPair& p : pairs) std::fprintf(f, "%d, %d\n", p.QueryPoint, p.CandidatePoint);
+    // "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54; with distances
+    // "q, c, dist\n", the three-column form results/scripts/neighbor_tables.py:102-115 also reads
+    if (dist.size() == pairs.size() && !pairs.empty())
+        for (size_t i = 0; i < pairs.size(); ++i)
+            std::fprintf(f, "%d, %d, %.7g\n", pairs[i].QueryPoint, pairs[i].CandidatePoint, dist[i]);
+    else
+        for (const FastedPair& p : pairs) std::fprintf(f, "%d, %d\n", p.QueryPoint, p.CandidatePoint);
     std::fclose(f);
 }
 
@@ -375,6 +388,7 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
 
     FastedJoinStats st{};
     std::vector<FastedPair> pairs;
+    std::vector<float> distances;
     try {
         const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
         join_on_device(all, all, true, tb.dPad, epsilon, dPairs, maxPairs, FASTED_SORT_PAIRS, nullptr, &st);
@@ -386,6 +400,17 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
         pairs.resize((size_t)st.pairsStored);
         if (st.pairsStored)
             HIP_CHECK(hipMemcpy(pairs.data(), dPairs, pairs.size() * sizeof(FastedPair), hipMemcpyDeviceToHost));
+        if (savePairs && save_distances() && st.pairsStored) {
+            float* dDist = nullptr;
+            HIP_CHECK(hipMalloc(&dDist, pairs.size() * sizeof(float)));
+            hipError_t e = fasted::launch_pair_distances(g_res.dPoints, tb.dPad, tb.n, g_res.dPoints, tb.dPad, tb.n,
+                                                         tb.dPad, dPairs, st.pairsStored, dDist, nullptr);
+            distances.resize(pairs.size());
+            if (e == hipSuccess)
+                e = hipMemcpy(distances.data(), dDist, distances.size() * sizeof(float), hipMemcpyDeviceToHost);
+            (void)hipFree(dDist);
+            HIP_CHECK(e);
+        }
     } catch (...) {
         (void)hipFree(dPairs);
         throw;
@@ -394,7 +419,7 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
     if (savePairs) {
         const std::string path = output_dir() + "/" + datasetName + "_" + std::to_string(epsilon) + ".pairs";
         std::cout << "Output file is: " << path << std::endl;
-        write_pairs_text(path, pairs);
+        write_pairs_text(path, pairs, distances);
     }
     const double totalTime = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
     const float kernelSec = (st.sumSquaredMs + st.joinMs) / 1000.0f;
@@ -556,6 +581,21 @@ int fasted_join_device(const void* d_queries, long long n_queries, long long ld_
     });
 }
 
+int fasted_pair_distances_device(const void* d_queries, long long n_queries, long long ld_queries,
+                                 const void* d_candidates, long long n_candidates, long long ld_candidates, int d,
+                                 const FastedPair* d_pairs, unsigned long long count, float* d_distances, void* stream) {
+    return guarded([&] {
+        if (!d_queries || !d_candidates) throw std::invalid_argument("points pointer is null");
+        if (count > 0 && (!d_pairs || !d_distances)) throw std::invalid_argument("pair or distance buffer is null");
+        validate_shape(n_queries, d, ld_queries);
+        validate_shape(n_candidates, d, ld_candidates);
+        HIP_CHECK(fasted::launch_pair_distances(d_queries, ld_queries, (int)n_queries, d_candidates, ld_candidates,
+                                                (int)n_candidates, round_up(d, fasted::kSlabK), d_pairs, count,
+                                                d_distances, static_cast<hipStream_t>(stream)));
+        HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    });
+}
+
 int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream) {
     return guarded([&] {
         if (!d_points || !d_sums) throw std::invalid_argument("null pointer");
@@ -693,6 +733,8 @@ const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad) {
 }
 
 void fasted_set_output_dir(const char* dir) { g_outDir = dir ? dir : ""; }
+
+void fasted_set_save_distances(int enabled) { g_saveDistances = enabled != 0; }
 
 const char* fasted_last_error(void) { return g_error.c_str(); }
 

@@ -46,4 +46,10 @@ hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
 // Row-major sort of `count` stored pairs (pair_sort.hip).
 hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream);
 
+// out[i] = Euclidean distance of pair i (FP32 sum of squared differences over dPad dimensions); NaN for a
+// pair that names a point outside [0, nQ) x [0, nC).
+hipError_t launch_pair_distances(const void* queries, long long ldQ, int nQ, const void* candidates, long long ldC,
+                                 int nC, int dPad, const void* pairs, unsigned long long count, float* out,
+                                 hipStream_t stream);
+
 }  // namespace fasted

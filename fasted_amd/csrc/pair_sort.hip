@@ -1,4 +1,5 @@
-// pair_sort.hip -- row-major ordering of the stored pairs on the device.
+// pair_sort.hip -- what happens to the stored pairs on the device after the join: the row-major
+// ordering, and the optional distance of every pair.
 //
 // The reference sorts its pair buffer with thrust::sort and Pair::operator< (query index,
 // then candidate index; source/pair.cuh:39-45,151-158).  A pair is 8 bytes with the query
@@ -19,6 +20,41 @@ __global__ void rotate_pairs_kernel(const unsigned long long* __restrict__ in, u
     for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
         const unsigned long long v = in[i];
         out[i] = (v << 32) | (v >> 32);
+    }
+}
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Euclidean distance of every listed pair, sum of squared differences in FP32 (no cancellation, unlike
+// the expansion the join itself tests).  16 lanes share a pair: 16-byte chunks of both rows, strided.
+// Pairs that name a point outside its set get NaN.
+__global__ void __launch_bounds__(256) pair_distances_kernel(const u32x4* __restrict__ ptsQ, long long ldQ16, int nQ,
+                                                             const u32x4* __restrict__ ptsC, long long ldC16, int nC,
+                                                             int chunksPerRow, const int2* __restrict__ pairs,
+                                                             unsigned long long count, float* __restrict__ out) {
+    const int sub = threadIdx.x & 15;
+    const unsigned long long groups = ((unsigned long long)gridDim.x * blockDim.x) >> 4;
+    for (unsigned long long g = ((unsigned long long)blockIdx.x * blockDim.x + threadIdx.x) >> 4; g < count; g += groups) {
+        const int2 pr = pairs[g];
+        const bool valid = pr.x >= 0 && pr.x < nQ && pr.y >= 0 && pr.y < nC;
+        float acc = 0.0f;
+        if (valid) {
+            const u32x4* a = ptsQ + (long long)pr.x * ldQ16;
+            const u32x4* b = ptsC + (long long)pr.y * ldC16;
+            for (int c = sub; c < chunksPerRow; c += 16) {
+                const half8 x = __builtin_bit_cast(half8, a[c]);
+                const half8 y = __builtin_bit_cast(half8, b[c]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float diff = (float)x[e] - (float)y[e];
+                    acc = __builtin_fmaf(diff, diff, acc);
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (sub == 0) out[g] = valid ? __builtin_sqrtf(acc) : __builtin_nanf("");
     }
 }
 
@@ -52,6 +88,17 @@ hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream
     if (temp) (void)hipFree(temp);
     (void)hipFree(alt);
     return e;
+}
+
+hipError_t launch_pair_distances(const void* queries, long long ldQ, int nQ, const void* candidates, long long ldC,
+                                 int nC, int dPad, const void* pairs, unsigned long long count, float* out,
+                                 hipStream_t stream) {
+    if (count == 0) return hipSuccess;
+    const unsigned long long blocks = (count * 16 + 255) / 256;
+    pair_distances_kernel<<<dim3((unsigned)(blocks > 16384ull ? 16384ull : blocks)), dim3(256), 0, stream>>>(
+        static_cast<const u32x4*>(queries), ldQ / 8, nQ, static_cast<const u32x4*>(candidates), ldC / 8, nC, dPad / 8,
+        static_cast<const int2*>(pairs), count, out);
+    return hipGetLastError();
 }
 
 }  // namespace fasted

@@ -120,6 +120,12 @@ def load_findpairs(path: str = None):
     lib.fasted_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_longlong, c.c_void_p, c.c_longlong, c.c_longlong,
                                        c.c_int, c.c_double, c.c_void_p, c.c_void_p, c.c_void_p, c.c_ulonglong, c.c_uint,
                                        c.c_void_p, c.POINTER(FastedJoinStats)]
+    lib.fasted_pair_distances_device.restype = c.c_int
+    lib.fasted_pair_distances_device.argtypes = [c.c_void_p, c.c_longlong, c.c_longlong, c.c_void_p, c.c_longlong,
+                                                 c.c_longlong, c.c_int, c.c_void_p, c.c_ulonglong, c.c_void_p,
+                                                 c.c_void_p]
+    lib.fasted_set_save_distances.restype = None
+    lib.fasted_set_save_distances.argtypes = [c.c_int]
     lib.fasted_sum_squared_device.restype = c.c_int
     lib.fasted_sum_squared_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_void_p, c.c_void_p]
     lib.fasted_raster_coord.restype = c.c_int
@@ -223,6 +229,14 @@ def count_pairs(epsilon):
     found, secs = ctypes.c_ulonglong(), ctypes.c_double()
     _check(lib, lib.fasted_count_pairs(float(epsilon), ctypes.byref(found), ctypes.byref(secs)))
     return found.value, secs.value
+
+
+def pair_distances_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates, d,
+                          pairs_ptr, count, distances_ptr, stream=None):
+    """FP32 Euclidean distance of every listed pair, on raw device pointers."""
+    lib = load_findpairs()
+    _check(lib, lib.fasted_pair_distances_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates,
+                                                 ld_candidates, d, pairs_ptr, count, distances_ptr, stream))
 
 
 def find_epsilon(target_selectivity, initial_epsilon=0.0):

@@ -136,6 +136,15 @@ int fasted_join_device(const void* d_queries, long long n_queries, long long ld_
                        float* d_sums_candidates, FastedPair* d_pairs, unsigned long long cap, unsigned flags,
                        void* stream, FastedJoinStats* stats);
 
+/* Euclidean distance of each of `count` listed pairs (QueryPoint indexes the queries, CandidatePoint the
+ * candidates; pass the same set twice for the output of a self-join): d_distances[i] in FP32, formed as
+ * the sum of squared differences, NaN for a pair that names a point outside its set.  The reference never
+ * reports distances, but its neighbour-table script reads an optional third column "q, c, dist"
+ * (results/scripts/neighbor_tables.py:102-115); this fills it. */
+int fasted_pair_distances_device(const void* d_queries, long long n_queries, long long ld_queries,
+                                 const void* d_candidates, long long n_candidates, long long ld_candidates, int d,
+                                 const FastedPair* d_pairs, unsigned long long count, float* d_distances, void* stream);
+
 /* Squared norms only: sums[i] = sum_k x_ik^2 in FP32.  Replaces
  * SumSqd::ComputeSquaredSums (source/sumSquared.cuh:84-118). */
 int fasted_sum_squared_device(const void* d_points, long long n, int d, long long ld, float* d_sums, void* stream);
@@ -185,6 +194,11 @@ const char* fasted_resident_name(void);
 /* Where `savePairs` writes "<name>_<epsilon>.pairs" (default: $FASTED_PAIRS_DIR or ".").
  * The reference hard-codes a cluster path at source/main.cu:214-215. */
 void fasted_set_output_dir(const char* dir);
+
+/* With a non-zero argument (or $FASTED_PAIRS_DISTANCES set) `savePairs` writes "q, c, dist" lines, the
+ * three-column form results/scripts/neighbor_tables.py:102-115 accepts; default "q, c" as
+ * source/pair.cuh:51-54. */
+void fasted_set_save_distances(int enabled);
 
 const char* fasted_last_error(void);
 const char* fasted_version(void);

@@ -141,3 +141,28 @@ def test_experiment_sweep_reproduces_the_reference_result_records(lib, tmp_path)
         assert r["results"]["paddedProblemShape"]["k"] == g["results"]["paddedProblemShape"]["k"]
         assert r["results"]["TFLOPS"] > 0
     lib.releaseResources()
+
+
+def test_pairs_file_with_the_distance_column(lib, tmp_path):
+    """Opt-in third column "q, c, dist" (the form results/scripts/neighbor_tables.py:102-115 parses)."""
+    rng = np.random.default_rng(5)
+    vals = np.round(rng.random((700, 70)), 6)
+    csv = tmp_path / "dist700.csv"
+    write_csv(csv, vals)
+    bits = oracle.quantize(vals)
+    eps = datasets.epsilon_for_neighbours(bits, 8)
+    lib.fasted_set_output_dir(str(tmp_path).encode())
+    lib.fasted_set_save_distances(1)
+    try:
+        r = lib.runFromFile(str(csv).encode(), eps, True)
+    finally:
+        lib.fasted_set_save_distances(0)
+    lines = (tmp_path / ("dist700_%f.pairs" % eps)).read_text().splitlines()
+    assert len(lines) == r.pairsStored
+    parsed = [re.fullmatch(r"(\d+), (\d+)(, (.+))?", line).group(1, 2, 4) for line in lines]
+    got = np.array([[int(q), int(c)] for q, c, _ in parsed], dtype=np.int32)
+    dist = np.array([float(x) for _, _, x in parsed])
+    assert np.allclose(dist, oracle.pair_distances_f64(bits, got), rtol=1e-5, atol=1e-6)
+    assert (dist <= eps * (1 + 1e-3)).all()
+    lib.releaseResources()
+    lib.fasted_set_output_dir(b"")

@@ -260,3 +260,38 @@ def test_blocked_join_overflow_is_soft(fasted):
     part, found = fasted.self_join_blocked(bits, eps, 512, cap=cap)
     assert found == found_whole and len(part) == cap
     assert np.array_equal(part, whole[:cap])  # row-major prefix: the first query blocks come first
+
+
+def test_pair_distances_match_fp64(fasted):
+    """Distance column of a pair list: FP32 sum of squared differences against the FP64 checker; every
+    reported pair lies within epsilon (up to the band); a pair naming a missing point yields NaN."""
+    import torch
+
+    n, d = 1500, 192
+    bits = datasets.uniform_bytes(n, d, seed=77)
+    eps = datasets.epsilon_for_neighbours(bits, 12)
+    got, st, _ = device_join(fasted, bits, eps)
+    want = oracle.pair_distances_f64(bits, got)
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    pairs = torch.from_numpy(np.vstack([got, [[n, 0]], [[0, -1]]]).astype(np.int32)).cuda()
+    dist = torch.full((len(got) + 2,), -1.0, dtype=torch.float32, device="cuda")
+    fasted.pair_distances_device(pts.data_ptr(), n, d, pts.data_ptr(), n, d, d, pairs.data_ptr(), len(got) + 2,
+                                 dist.data_ptr())
+    host = dist.cpu().numpy()
+    assert np.isnan(host[-2:]).all()
+    assert np.allclose(host[:-2], want, rtol=2e-6, atol=1e-6)  # FP32 accumulation of <= 192 exact-ish terms
+    assert (host[:-2] <= eps * (1 + 1e-3)).all()
+    self_pairs = got[:, 0] == got[:, 1]
+    assert (host[:-2][self_pairs] == 0).all()
+
+    # two different sets, ragged sizes and row strides
+    nq, nc = 300, 1000
+    q_bits, c_bits = bits[:nq], bits[n - nc:]
+    some = np.array([[0, 0], [299, 999], [17, 503]], dtype=np.int32)
+    qd, cd = (torch.from_numpy(b.view(np.int16).copy()).cuda() for b in (q_bits, c_bits))
+    out = torch.empty(3, dtype=torch.float32, device="cuda")
+    fasted.pair_distances_device(qd.data_ptr(), nq, d, cd.data_ptr(), nc, d, d, torch.from_numpy(some).cuda().data_ptr(), 3,
+                                 out.data_ptr())
+    both = np.vstack([q_bits, c_bits])
+    want2 = oracle.pair_distances_f64(both, some + np.array([0, nq], dtype=np.int32))
+    assert np.allclose(out.cpu().numpy(), want2, rtol=2e-6)
