@@ -101,7 +101,8 @@ void validate_shape(long long n, int d, long long ld) {
     const long long dPad = round_up(d, fasted::kSlabK);
     if (ld % 8 != 0) throw std::invalid_argument("row stride must be a multiple of 8 halves (16 bytes)");
     if (ld < dPad) throw std::invalid_argument("row stride must cover the dimensionality rounded up to 64");
-    if ((ld / 8) * fasted::kTile >= (1ll << 31)) throw std::invalid_argument("row stride too large");
+    // the kernel addresses a tile's rows with 32-bit byte offsets from the tile's first row
+    if (ld * 2 * fasted::kTile >= (1ll << 32)) throw std::invalid_argument("row stride too large");
 }
 
 // One side of a join: `n` FP16 rows of `d` dimensions, row stride `ld` halves.

@@ -130,9 +130,12 @@ def test_raw_entry_rejects_bad_arguments_without_touching_a_gpu(lib):
     st = fp.FastedJoinStats()
     assert lib.fasted_self_join_device(None, 10, 64, 64, 0.1, None, None, 0, 0, None, ctypes.byref(st)) != 0
     buf = (ctypes.c_uint16 * 64)()
-    for n, d, ld in [(0, 64, 64), (10, 0, 64), (10, 64, 60), (10, 100, 64)]:
+    for n, d, ld in [(0, 64, 64), (10, 0, 64), (10, 64, 60), (10, 100, 64), (10, 64, 1 << 23), (2 ** 31 - 1, 64, 64)]:
         rc = lib.fasted_self_join_device(ctypes.addressof(buf), n, d, ld, 0.1, None, None, 0, 0, None, ctypes.byref(st))
         assert rc != 0 and lib.fasted_last_error()
+    assert lib.fasted_self_join_blocked(ctypes.addressof(buf), 10, 8, 0.1, 0, None, 0, None, None) != 0
+    assert b"block" in lib.fasted_last_error()
+    assert lib.fasted_pair_distances_device(None, 1, 64, None, 1, 64, 64, None, 0, None, None) != 0
 
 
 # ---------------------------------------------------------------- tile queues (host mirror)
