@@ -92,7 +92,7 @@ def calibrate_epsilon(torch, pts, neighbours, sample=4096, seed=4242):
     return math.sqrt(eps2)
 
 
-def parity_sample(torch, pts, eps, pairs, stored, rows=256, seed=7, band=1e-3):
+def parity_sample(torch, pts, eps, pairs, stored, rows=1024, seed=7, band=1e-3):
     """Pair-set check of `rows` seeded query rows against FP64 distances to all points (torch FP64 on
     the device, outside the timed region): pairs that disagree with FP64, how many of them lie outside
     the relative `band` around epsilon (must be 0), and the largest relative distance error."""

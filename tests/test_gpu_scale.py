@@ -95,17 +95,17 @@ def run_config(env, name, n=None, sample_rows=256, oracle_rows=0):
 
 
 def test_config2_low_dim_100k_x_128(env):
-    run_config(env, "c2", sample_rows=512, oracle_rows=64)
+    run_config(env, "c2", sample_rows=1024, oracle_rows=64)
 
 
 def test_config4_clustered_500k_x_960(env):
-    run_config(env, "c4", sample_rows=256, oracle_rows=4)
+    run_config(env, "c4", sample_rows=1024, oracle_rows=4)
 
 
 def test_config5_output_heavy_2m_x_384(env):
-    st = run_config(env, "c5", sample_rows=128)
+    st = run_config(env, "c5", sample_rows=1024)
     assert st.pairsFound > 2e8  # the output-heavy case really is output heavy
 
 
 def test_config3_headline_1m_x_4096(env):
-    run_config(env, "c3", sample_rows=256)
+    run_config(env, "c3", sample_rows=1024)
