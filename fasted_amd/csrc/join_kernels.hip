@@ -517,12 +517,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             if (mirror) mine *= 2;
             if (__builtin_amdgcn_ballot_w64(mine != 0) != 0ull) {
                 // wave-level compaction: inclusive prefix sum of per-lane counts, one reservation
+                // (data-parallel-primitive moves inside the vector ALU: shifts within rows of 16 lanes, then the
+                // last lane of row 0/2 added to row 1/3, then lane 31 to the upper half)
                 int incl = mine;
-#pragma unroll
-                for (int off = 1; off < 64; off <<= 1) {
-                    const int v = __builtin_amdgcn_ds_bpermute((ln - off) << 2, incl);
-                    if (ln >= off) incl += v;
-                }
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x111, 0xf, 0xf, false);  // row_shr:1
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x112, 0xf, 0xf, false);  // row_shr:2
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x114, 0xf, 0xf, false);  // row_shr:4
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x118, 0xf, 0xf, false);  // row_shr:8
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+                incl += __builtin_amdgcn_update_dpp(0, incl, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
                 const unsigned total = (unsigned)__builtin_amdgcn_readlane(incl, 63);
                 // reserve room in the staging area (LDS atomic); what does not fit goes straight
                 // to the global list with a reservation of this wave's own
