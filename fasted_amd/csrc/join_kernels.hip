@@ -172,9 +172,8 @@ struct JoinParams {
 //     a >= -eps^2/2,
 // one threshold for every element, exact in FP32 (the scaling by 2 is exact), and symmetric in q and c
 // like the reference's.  Screening, 1/3 VALU op per element: the maximum of the lane's 128 elements
-// against the threshold; a wave in which no lane has a hit is done.  Otherwise the blocks are screened
-// one by one (maximum of the lane's 4 rows, wave-wide ballot) and the blocks with a hit yield their
-// per-element bits.
+// against the threshold; a wave in which no lane has a hit is done.  Otherwise every element yields its
+// bit, branch-free.
 //
 // kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; self pairs are
 // forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
@@ -206,28 +205,21 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
             const int fi = fp * 2 + h;
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj) {
-                bool look = kEdge;
-                if (!kEdge) {
-                    const floatx4 f = acc[fi][fj];
-                    const float best = __builtin_fmaxf(__builtin_fmaxf(f[0], f[1]), __builtin_fmaxf(f[2], f[3]));
-                    look = __builtin_amdgcn_ballot_w64(best >= thr) != 0ull;
-                }
-                if (look) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        bool hit = acc[fi][fj][r] >= thr;
-                        if (kEdge) {
-                            const int q = qBase + fi * 16 + quad * 4 + r;
-                            hit = (hit || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
-                        }
+                for (int r = 0; r < 4; ++r) {
+                    if (kEdge) {
+                        const int q = qBase + fi * 16 + quad * 4 + r;
+                        const bool hit =
+                            (acc[fi][fj][r] >= thr || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
                         m = (m << 1) | (hit ? 1u : 0u);
+                    } else {
+                        // two instructions per element: the sign of acc - thr (set = no hit) is shifted in
+                        m = __builtin_amdgcn_alignbit(m, __builtin_bit_cast(unsigned, acc[fi][fj][r] - thr), 31);
                     }
-                } else {
-                    m <<= 4;
                 }
             }
         }
-        mask[fp] = m;
+        mask[fp] = kEdge ? m : ~m;
     }
 }
 
