@@ -295,3 +295,30 @@ def test_pair_distances_match_fp64(fasted):
     both = np.vstack([q_bits, c_bits])
     want2 = oracle.pair_distances_f64(both, some + np.array([0, nq], dtype=np.int32))
     assert np.allclose(out.cpu().numpy(), want2, rtol=2e-6)
+
+
+def test_caller_stream_and_repeatability(fasted):
+    """The device entry on a stream of the caller's: work queued on that stream before the call is seen,
+    the call returns with the stream drained, and repeated calls give the same sorted list."""
+    import torch
+
+    n, d = 3000, 128
+    bits = datasets.uniform_bytes(n, d, seed=99)
+    eps = datasets.epsilon_for_neighbours(bits, 10)
+    want, st_want, _ = device_join(fasted, bits, eps)
+    stream = torch.cuda.Stream()  # default priority
+    cap = 300 * n
+    host = torch.from_numpy(bits.view(np.int16).copy()).pin_memory()
+    with torch.cuda.stream(stream):
+        pts = torch.empty((n, d), dtype=torch.int16, device="cuda")
+        pts.copy_(host, non_blocking=True)  # still in flight on `stream` when the join is queued behind it
+        pairs = torch.full((cap, 2), -1, dtype=torch.int32, device="cuda")
+        runs = []
+        for _ in range(3):
+            st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, stream=stream.cuda_stream)
+            assert stream.query()  # nothing left on the stream: the call synchronised it
+            runs.append(pairs[: st.pairsStored].cpu().numpy().copy())
+    torch.cuda.synchronize()
+    assert st.pairsFound == st_want.pairsFound
+    for got in runs:
+        assert np.array_equal(got, want)
