@@ -1,5 +1,6 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/reference_loader.json from the REFERENCE's own host data loader.
+"""Writes tests/golden/reference_loader.json from the REFERENCE's own host data loader, and
+tests/golden/speed_results_records.json from the result files the reference holds.
 
 The reference's DataLoader/*.hpp (ExponentialPointGenerator, FilePointGenerator,
 PointListBuilder<half>, half.hpp) are compiled in place into oracle/_ref/libfasted_ref.so by
@@ -69,6 +70,27 @@ def main():
     with open(os.path.join(HERE, "reference_loader.json"), "w") as f:
         json.dump(out, f, indent=1)
     print("wrote reference_loader.json")
+    speed_result_records()
+
+
+def speed_result_records(reference="/root/reference"):
+    """Records of the reference's stored experiment results (plain JSON data): the cells of the size x
+    dimensionality sweep that are small enough to re-run in a test and whose pair counts do not depend on
+    the A100's rounding (D <= 256: exactly the self pairs), plus one record of the selectivity
+    experiment for its schema."""
+    base = os.path.join(reference, "results", "speed_results")
+    with open(os.path.join(base, "ExpoDataSpeedVsSize_OnDemandRasterizer.json")) as f:
+        sweep = json.load(f)
+    with open(os.path.join(base, "selectivityVsSpeed.json")) as f:
+        selectivity = json.load(f)
+    keep = [r for r in sweep if r["iteration"] == 0 and r["results"]["inputProblemShape"]["m"] <= 2200
+            and r["results"]["inputProblemShape"]["k"] <= 256]
+    out = {"source": "results/speed_results/ExpoDataSpeedVsSize_OnDemandRasterizer.json (records with iteration 0, "
+                     "N <= 2200, D <= 256) and the first record of selectivityVsSpeed.json",
+           "sweep": keep, "selectivity_record": selectivity[0]}
+    with open(os.path.join(HERE, "speed_results_records.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("wrote speed_results_records.json")
 
 
 if __name__ == "__main__":
