@@ -112,15 +112,28 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
     float acc = 0.0f;
     if (row < n) {
         const u32x4* p = pts + row * ld16;
-        for (int c = sub; c < chunksPerRow; c += lanesPerRow) {
-            u32x4 v = p[c];
-            half8 h = __builtin_bit_cast(half8, v);
+        auto square_add = [](u32x4 v, float a) {
+            const half8 h = __builtin_bit_cast(half8, v);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float x = (float)h[e];
-                acc = __builtin_fmaf(x, x, acc);
+                const float x = (float)h[e];
+                a = __builtin_fmaf(x, x, a);
             }
+            return a;
+        };
+        // four independent 16-byte loads in flight per lane (one alone leaves the memory pipe idle
+        // for most of its latency), four partial sums
+        float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        int c = sub;
+        for (; c + 3 * lanesPerRow < chunksPerRow; c += 4 * lanesPerRow) {
+            const u32x4 v0 = p[c], v1 = p[c + lanesPerRow], v2 = p[c + 2 * lanesPerRow], v3 = p[c + 3 * lanesPerRow];
+            part[0] = square_add(v0, part[0]);
+            part[1] = square_add(v1, part[1]);
+            part[2] = square_add(v2, part[2]);
+            part[3] = square_add(v3, part[3]);
         }
+        for (; c < chunksPerRow; c += lanesPerRow) part[0] = square_add(p[c], part[0]);
+        acc = (part[0] + part[1]) + (part[2] + part[3]);
     }
     for (int off = lanesPerRow >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
     if (sub == 0 && row < n) sums[row] = acc;
