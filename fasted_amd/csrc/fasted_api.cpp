@@ -13,6 +13,7 @@
 #include <climits>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <fstream>
 #include <iostream>
 #include <string>
@@ -182,6 +183,47 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     }
 }
 
+// Host rows of `rowBytes` bytes -> device rows of `pitch` bytes (pitch >= rowBytes; the bytes past rowBytes
+// are written as zeros).  Rows that are already contiguous go up in one copy; otherwise they are packed
+// into two pinned staging buffers in turn, so that packing one chunk overlaps the transfer of the other
+// (a strided 2-D copy from pageable memory moves row by row, at about 1 GB/s).
+void upload_rows(void* dst, size_t pitch, const void* src, size_t rowBytes, size_t rows, hipStream_t stream) {
+    if (rows == 0) return;
+    if (rowBytes == pitch) {
+        HIP_CHECK(hipMemcpyAsync(dst, src, rows * pitch, hipMemcpyHostToDevice, stream));
+        return;
+    }
+    const size_t chunkRows = std::max<size_t>(1, std::min(rows, ((size_t)32 << 20) / pitch));
+    struct Staging {
+        void* buf[2] = {nullptr, nullptr};
+        hipEvent_t done[2] = {nullptr, nullptr};
+        ~Staging() {
+            for (int i = 0; i < 2; ++i) {
+                if (buf[i]) (void)hipHostFree(buf[i]);
+                if (done[i]) (void)hipEventDestroy(done[i]);
+            }
+        }
+    } st;
+    for (int i = 0; i < 2; ++i) {
+        HIP_CHECK(hipHostMalloc(&st.buf[i], chunkRows * pitch, hipHostMallocDefault));
+        HIP_CHECK(hipEventCreateWithFlags(&st.done[i], hipEventDisableTiming));
+    }
+    int slot = 0;
+    for (size_t r0 = 0; r0 < rows; r0 += chunkRows, slot ^= 1) {
+        const size_t count = std::min(chunkRows, rows - r0);
+        HIP_CHECK(hipEventSynchronize(st.done[slot]));  // the transfer that last read this buffer is over
+        char* out = static_cast<char*>(st.buf[slot]);
+        const char* in = static_cast<const char*>(src) + r0 * rowBytes;
+        for (size_t r = 0; r < count; ++r) {
+            std::memcpy(out + r * pitch, in + r * rowBytes, rowBytes);
+            std::memset(out + r * pitch + rowBytes, 0, pitch - rowBytes);
+        }
+        HIP_CHECK(hipMemcpyAsync(static_cast<char*>(dst) + r0 * pitch, out, count * pitch, hipMemcpyHostToDevice, stream));
+        HIP_CHECK(hipEventRecord(st.done[slot], stream));
+    }
+    HIP_CHECK(hipStreamSynchronize(stream));  // the staging buffers go away with this frame
+}
+
 // Self-join of a host-resident dataset that is streamed through the device in blocks of `blockRows`
 // points: for every query block (held on the device) every candidate block is uploaded in turn, on a
 // copy stream, while the join of the block before it runs.  The pairs of one query block are appended
@@ -223,11 +265,6 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
     float* qSums = static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)));
     float* cSums[2] = {static_cast<float*>(dev.alloc((size_t)rows * sizeof(float))),
                        static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)))};
-    if (dPad != d) {  // the columns d..dPad are never written again and must read as zeros
-        HIP_CHECK(hipMemset(qBlock, 0, blockBytes));
-        HIP_CHECK(hipMemset(cBlock[0], 0, blockBytes));
-        HIP_CHECK(hipMemset(cBlock[1], 0, blockBytes));
-    }
     // pair buffer of one query block: rows*256 records as the reference sizes its buffer per point
     // (source/findPairs.cuh:644-647), shrunk to half of what is free (the sort needs as much again)
     unsigned long long devCap = std::min<unsigned long long>((unsigned long long)rows * 256ull, cap);
@@ -239,8 +276,7 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
 
     auto block_rows = [&](long long b) { return std::min<long long>(rows, n - b * rows); };
     auto upload = [&](void* dst, long long b, hipStream_t s) {
-        HIP_CHECK(hipMemcpy2DAsync(dst, pitch, points + (size_t)b * rows * d, (size_t)d * 2, (size_t)d * 2,
-                                   (size_t)block_rows(b), hipMemcpyHostToDevice, s));
+        upload_rows(dst, pitch, points + (size_t)b * rows * d, (size_t)d * 2, (size_t)block_rows(b), s);
     };
     unsigned long long foundAll = 0, storedAll = 0;
     const float eps2 = static_cast<float>(epsilon * epsilon);
@@ -620,9 +656,8 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
         try {
             const size_t pitch = (size_t)dPad * 2;
             HIP_CHECK(hipMalloc(&dPoints, (size_t)n * pitch));
-            if (dPad != d) HIP_CHECK(hipMemset(dPoints, 0, (size_t)n * pitch));
-            HIP_CHECK(hipMemcpy2D(dPoints, pitch, points, (size_t)d * 2, (size_t)d * 2, (size_t)n,
-                                  hipMemcpyHostToDevice));
+            upload_rows(dPoints, pitch, points, (size_t)d * 2, (size_t)n, nullptr);
+            HIP_CHECK(hipStreamSynchronize(nullptr));
             HIP_CHECK(hipMalloc(&dPairs, (size_t)(cap ? cap : 1) * sizeof(FastedPair)));
             FastedJoinStats st{};
             const PointSet all{dPoints, n, dPad, nullptr};
