@@ -574,8 +574,7 @@ Results runFromExponentialDataset(int size, int dimensionality, double lambda, d
     if (!quiet()) std::cout << "Running from a generated exponential dataset" << std::endl;
     return run_built(
         [&] {
-            fasted::ExponentialSource src(size, dimensionality, lambda, max);
-            return fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+            return fasted::build_exponential_table(size, dimensionality, lambda, max, fasted::kSlabK, fasted::kTile);
         },
         epsilon, savePairs);
 }
@@ -684,9 +683,8 @@ int fasted_self_join_blocked(const uint16_t* points, long long n, int d, double 
 
 int fasted_load_exponential_dataset(int size, int dimensionality, double lambda, double max) {
     return guarded([&] {
-        fasted::ExponentialSource src(size, dimensionality, lambda, max);
         g_res.drop_device();
-        g_res.table = fasted::build_point_table(src, fasted::kSlabK, fasted::kTile);
+        g_res.table = fasted::build_exponential_table(size, dimensionality, lambda, max, fasted::kSlabK, fasted::kTile);
     });
 }
 

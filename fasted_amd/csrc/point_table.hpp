@@ -9,11 +9,15 @@
 // Same seeds, same draw order, same double -> float -> half rounding, same padding rule,
 // same dataset names and the same error texts, so a caller sees the same dataset.
 #pragma once
+#include <algorithm>
 #include <cerrno>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
 #include <cstdlib>
+#include <condition_variable>
+#include <functional>
+#include <mutex>
 #include <fstream>
 #include <ios>
 #include <iterator>
@@ -124,6 +128,210 @@ inline PointTable build_point_table(PointSource& src, int dimMultiple, int point
     return t;
 }
 
+inline unsigned host_threads(const char* specificEnv) {
+    const char* env = std::getenv(specificEnv);
+    if (!env) env = std::getenv("FASTED_HOST_THREADS");
+    unsigned t = env ? static_cast<unsigned>(std::atoi(env)) : std::thread::hardware_concurrency();
+    if (t == 0) t = 1;
+    return t > 16 ? 16 : t;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The seeded exponential dataset, built by several threads, value for value what
+// build_point_table(ExponentialSource) gives.  What makes that possible: every candidate value of
+// std::exponential_distribution<double> over std::mt19937 consumes exactly two engine outputs
+// (std::generate_canonical<double, 53> with a 32-bit engine), whether it is then rejected or not, so
+// candidate i is a function of outputs 2i and 2i+1 alone and the dataset is the accepted candidates
+// in order.  One thread runs the engine (the only sequential part, 1 to 1.5 ns per output), the
+// others turn blocks of raw outputs into candidates (logarithm, range test, quantisation), and the
+// accepted values of each block are copied to their place once the blocks before it are counted.
+namespace detail {
+
+// The output stream of std::mt19937 (MT19937, 32 bit), produced a state block of 624 words at a time:
+// the same recurrence and tempering, written as plain loops over the block, about ten times faster than
+// one engine call per output.
+class Mt19937Stream {
+   public:
+    explicit Mt19937Stream(uint32_t seed) {
+        state_[0] = seed;
+        for (uint32_t i = 1; i < kWords; ++i) state_[i] = 1812433253u * (state_[i - 1] ^ (state_[i - 1] >> 30)) + i;
+    }
+    void generate(uint32_t* out, size_t count) {
+        while (count > 0) {
+            if (next_ == kWords) refill();
+            const size_t run = std::min<size_t>(count, kWords - next_);
+            std::memcpy(out, tempered_ + next_, run * sizeof(uint32_t));
+            out += run;
+            next_ += static_cast<uint32_t>(run);
+            count -= run;
+        }
+    }
+
+   private:
+    static constexpr uint32_t kWords = 624, kShift = 397;
+    static uint32_t mix(uint32_t upper, uint32_t lower) {
+        const uint32_t y = (upper & 0x80000000u) | (lower & 0x7fffffffu);
+        return (y >> 1) ^ ((lower & 1u) ? 0x9908b0dfu : 0u);
+    }
+    void refill() {
+        uint32_t i = 0;
+        for (; i < kWords - kShift; ++i) state_[i] = state_[i + kShift] ^ mix(state_[i], state_[i + 1]);
+        for (; i < kWords - 1; ++i) state_[i] = state_[i + kShift - kWords] ^ mix(state_[i], state_[i + 1]);
+        state_[kWords - 1] = state_[kShift - 1] ^ mix(state_[kWords - 1], state_[0]);
+        for (i = 0; i < kWords; ++i) {
+            uint32_t y = state_[i];
+            y ^= y >> 11;
+            y ^= (y << 7) & 0x9d2c5680u;
+            y ^= (y << 15) & 0xefc60000u;
+            y ^= y >> 18;
+            tempered_[i] = y;
+        }
+        next_ = 0;
+    }
+    uint32_t state_[kWords];
+    uint32_t tempered_[kWords];
+    uint32_t next_ = kWords;
+};
+
+// A few worker threads that run one job after another: start(body) has worker w call body(b) for the blocks
+// b = w, w + workers, ... < blocks; wait() returns when all of them are through.  (Threads are kept
+// because creating one per round costs more than a round's work.)
+class RoundPool {
+   public:
+    RoundPool(unsigned workers, size_t blocks) : workers_(workers), blocks_(blocks) {
+        for (unsigned w = 0; w < workers_; ++w) threads_.emplace_back([this, w] { loop(w); });
+    }
+    ~RoundPool() {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            stop_ = true;
+        }
+        wake_.notify_all();
+        for (auto& t : threads_) t.join();
+    }
+    void start(std::function<void(size_t)> body) {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            body_ = std::move(body);
+            pending_ = workers_;
+            ++round_;
+        }
+        wake_.notify_all();
+    }
+    void wait() {
+        std::unique_lock<std::mutex> lock(mutex_);
+        done_.wait(lock, [this] { return pending_ == 0; });
+    }
+
+   private:
+    void loop(unsigned w) {
+        unsigned long long seen = 0;
+        for (;;) {
+            std::function<void(size_t)> body;
+            {
+                std::unique_lock<std::mutex> lock(mutex_);
+                wake_.wait(lock, [&] { return stop_ || round_ != seen; });
+                if (stop_) return;
+                seen = round_;
+                body = body_;
+            }
+            for (size_t b = w; b < blocks_; b += workers_) body(b);
+            std::lock_guard<std::mutex> lock(mutex_);
+            if (--pending_ == 0) done_.notify_all();
+        }
+    }
+    unsigned workers_;
+    size_t blocks_;
+    std::vector<std::thread> threads_;
+    std::mutex mutex_;
+    std::condition_variable wake_, done_;
+    std::function<void(size_t)> body_;
+    unsigned pending_ = 0;
+    unsigned long long round_ = 0;
+    bool stop_ = false;
+};
+
+// libstdc++'s generate_canonical<double, 53>(mt19937) followed by exponential_distribution<double>
+inline double exponential_from_outputs(uint32_t first, uint32_t second, double lambda) {
+    double sum = static_cast<double>(first) * 1.0;
+    sum += static_cast<double>(second) * 4294967296.0;
+    double u = sum / 18446744073709551616.0;
+    if (u >= 1.0) u = std::nextafter(1.0, 0.0);
+    return -std::log(1.0 - u) / lambda;
+}
+
+}  // namespace detail
+
+inline PointTable build_exponential_table(int numPoints, int numDims, double lambda, double maxValue, int dimMultiple,
+                                          int pointMultiple, unsigned threads = 0) {
+    if (threads == 0) threads = host_threads("FASTED_GEN_THREADS");
+    const unsigned long long total = numPoints > 0 && numDims > 0 ? 1ull * numPoints * numDims : 0ull;
+    if (threads < 2 || total < (1ull << 20)) {  // small or degenerate: the plain sequential builder
+        ExponentialSource src(numPoints, numDims, lambda, maxValue);
+        return build_point_table(src, dimMultiple, pointMultiple);
+    }
+    PointTable t;
+    t.name = ExponentialSource(numPoints, numDims, lambda, maxValue).name();
+    t.n = numPoints;
+    t.d = numDims;
+    t.dPad = round_up_to(numDims, dimMultiple);
+    t.nPad = round_up_to(numPoints, pointMultiple);
+    t.bits.assign(static_cast<size_t>(t.nPad) * static_cast<size_t>(t.dPad), 0);
+
+    constexpr size_t kBlock = 1u << 15;  // candidates per block
+    const unsigned workers = threads - 1;  // one thread runs the engine
+    const size_t roundBlocks = static_cast<size_t>(workers) * 4;
+    std::vector<uint32_t> raw[2];
+    raw[0].resize(2 * kBlock * roundBlocks);
+    raw[1].resize(2 * kBlock * roundBlocks);
+    std::vector<uint16_t> values(kBlock * roundBlocks);
+    std::vector<size_t> counts(roundBlocks), offsets(roundBlocks);
+    detail::Mt19937Stream engine(ExponentialSource::kSeed);
+    auto fill = [&](std::vector<uint32_t>& out) { engine.generate(out.data(), out.size()); };
+    detail::RoundPool pool(workers, roundBlocks);
+    fill(raw[0]);
+    unsigned long long produced = 0;
+    int cur = 0;
+    while (produced < total) {
+        const uint32_t* const in = raw[cur].data();
+        pool.start([&, in](size_t b) {
+            const uint32_t* r = in + 2 * kBlock * b;
+            uint16_t* out = values.data() + kBlock * b;
+            size_t kept = 0;
+            for (size_t i = 0; i < kBlock; ++i) {
+                const double v = detail::exponential_from_outputs(r[2 * i], r[2 * i + 1], lambda);
+                if (v < 0.0 || v > maxValue) continue;  // redrawn by the sequential generator
+                out[kept++] = quantize_half(v);
+            }
+            counts[b] = kept;
+        });
+        fill(raw[cur ^ 1]);  // the engine runs ahead while the workers convert
+        pool.wait();
+        unsigned long long at = produced;
+        for (size_t b = 0; b < roundBlocks; ++b) {
+            offsets[b] = static_cast<size_t>(at);
+            at += counts[b];
+        }
+        pool.start([&](size_t b) {
+            unsigned long long j = offsets[b];
+            const uint16_t* src = values.data() + kBlock * b;
+            size_t left = counts[b];
+            while (left > 0 && j < total) {  // contiguous run inside one row of the padded table
+                const size_t row = static_cast<size_t>(j / numDims), col = static_cast<size_t>(j % numDims);
+                const size_t run = std::min<unsigned long long>({left, static_cast<unsigned long long>(numDims - col), total - j});
+                std::memcpy(t.bits.data() + row * t.dPad + col, src, run * sizeof(uint16_t));
+                src += run;
+                left -= run;
+                j += run;
+            }
+        });
+        pool.wait();
+        produced = at;
+        cur ^= 1;
+    }
+    return t;
+}
+
 // ---------------------------------------------------------------------------------------------
 // CSV files: one point per line, fields separated by `delimiter`, each field parsed like std::stod
 // (leading blanks skipped, trailing characters after the number ignored, no number -> error).  The
@@ -221,12 +429,7 @@ inline PointTable load_csv_table(const std::string& path, char delim, int dimMul
     t.nPad = round_up_to(t.n, pointMultiple);
     t.bits.assign(static_cast<size_t>(t.nPad) * static_cast<size_t>(t.dPad), 0);
 
-    if (threads == 0) {
-        const char* env = std::getenv("FASTED_CSV_THREADS");
-        threads = env ? static_cast<unsigned>(std::atoi(env)) : std::thread::hardware_concurrency();
-        if (threads == 0) threads = 1;
-        if (threads > 16) threads = 16;
-    }
+    if (threads == 0) threads = host_threads("FASTED_CSV_THREADS");
     if (static_cast<long long>(threads) > lines) threads = static_cast<unsigned>(lines);
     std::vector<detail::CsvError> errors(threads);
     auto work = [&](unsigned w) {

@@ -90,6 +90,21 @@ def test_exponential_dataset_equals_oracle_on_a_larger_case(lib):
     assert np.array_equal(bits[:n, :d], oracle.quantize(oracle.exponential_points(700, 200, 40.0, 10.0)))
 
 
+@pytest.mark.parametrize("n,d,lam,mx", [(3000, 400, 40.0, 10.0), (5000, 333, 10.0, 0.05), (2049, 1000, 40.0, 0.02)])
+def test_exponential_dataset_built_by_several_threads(lib, n, d, lam, mx, monkeypatch):
+    """Above 2^20 values the dataset is built by an engine thread and converter threads; the result is
+    the sequential generator's, value for value, also when most candidates are rejected (second and
+    third case: 61 % and 45 % fall outside [0, max]) and when rows straddle the blocks."""
+    want = oracle.quantize(oracle.exponential_points(n, d, lam, mx))
+    for threads in ("1", "3", "8"):
+        monkeypatch.setenv("FASTED_GEN_THREADS", threads)
+        assert lib.fasted_load_exponential_dataset(n, d, lam, mx) == 0
+        bits, got_n, got_d, name = fasted_amd.resident_points()
+        assert (got_n, got_d) == (n, d) and name == "Exponential_%d_%d_%f" % (n, d, lam)
+        assert np.array_equal(bits[:n, :d], want), threads
+        assert bits[n:].sum() == 0 and bits[:, d:].sum() == 0
+
+
 def test_csv_dataset_equals_reference_golden(lib):
     g = GOLDEN["csv"]
     assert lib.fasted_load_file(os.path.join(GOLDEN_DIR, g["file"]).encode()) == 0
