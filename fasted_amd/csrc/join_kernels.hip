@@ -451,8 +451,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 for (int fj = 0; fj < kFragCols; ++fj) {
                     if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, fj);
 #pragma unroll
-                    for (int fi = 0; fi < 4; ++fi)
+                    for (int fs = 0; fs < 4; ++fs) {
+                        const int fi = (fj & 1) ? 3 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -468,9 +470,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 for (int fj = 0; fj < kFragCols; ++fj) {
                     if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, 4 + fj);
 #pragma unroll
-                    for (int fi = 0; fi < 4; ++fi)
+                    for (int fs = 0; fs < 4; ++fs) {
+                        const int fi = (fj & 1) ? 3 - fs : fs;
                         acc[fi + 4][fj] =
                             __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
