@@ -184,9 +184,9 @@ struct JoinParams {
 // and the reference's test  s_q + s_c - 2 q.c <= eps^2  (source/warpMma.cuh:241-257) reads
 //     a >= -eps^2/2,
 // one threshold for every element, exact in FP32 (the scaling by 2 is exact), and symmetric in q and c
-// like the reference's.  Screening, 1/3 VALU op per element: the maximum of the lane's 128 elements
-// against the threshold; a wave in which no lane has a hit is done.  Otherwise every element yields its
-// bit, branch-free.
+// like the reference's.  Screening, about 1/2 VALU op per element: the maximum of the lane's 128 elements
+// (formed per row of blocks) against the threshold; a wave in which no lane has a hit is done.  Otherwise
+// the rows of blocks with a hit somewhere in the wave yield their per-element bits, branch-free.
 //
 // kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; self pairs are
 // forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
@@ -196,43 +196,69 @@ template <bool kEdge>
 __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const int (&cand)[kFragCols],
                                            int qBase, int quad, int nQ, int nC, int selfJoin, float thr,
                                            unsigned (&mask)[kFragRows / 2]) {
-    if (!kEdge) {
-        float best = acc[0][0][0];
+    if (kEdge) {
 #pragma unroll
-        for (int fi = 0; fi < kFragRows; ++fi)
+        for (int fp = 0; fp < kFragRows / 2; ++fp) {
+            unsigned m = 0;
 #pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj)
+            for (int h = 0; h < 2; ++h) {
+                const int fi = fp * 2 + h;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) best = __builtin_fmaxf(best, acc[fi][fj][r]);
-        if (__builtin_amdgcn_ballot_w64(best >= thr) == 0ull) {
+                for (int fj = 0; fj < kFragCols; ++fj) {
 #pragma unroll
-            for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
-            return;
+                    for (int r = 0; r < 4; ++r) {
+                        const int q = qBase + fi * 16 + quad * 4 + r;
+                        const bool hit =
+                            (acc[fi][fj][r] >= thr || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
+                        m = (m << 1) | (hit ? 1u : 0u);
+                    }
+                }
+            }
+            mask[fp] = m;
         }
+        return;
     }
+    // maximum of every row of blocks (16 elements per lane), then of all of them
+    float rowBest[kFragRows];
+#pragma unroll
+    for (int fi = 0; fi < kFragRows; ++fi) {
+        float best = acc[fi][0][0];
+#pragma unroll
+        for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) best = __builtin_fmaxf(best, acc[fi][fj][r]);
+        rowBest[fi] = best;
+    }
+    float best = rowBest[0];
+#pragma unroll
+    for (int fi = 1; fi < kFragRows; ++fi) best = __builtin_fmaxf(best, rowBest[fi]);
+    if (__builtin_amdgcn_ballot_w64(best >= thr) == 0ull) {
+#pragma unroll
+        for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
+        return;
+    }
+    // some lane has a hit: rows of blocks without one (wave-wide) are skipped, the others yield their
+    // bits, two instructions per element: the sign of acc - thr (set = no hit) is shifted in
+    unsigned long long rowHit[kFragRows];
+#pragma unroll
+    for (int fi = 0; fi < kFragRows; ++fi) rowHit[fi] = __builtin_amdgcn_ballot_w64(rowBest[fi] >= thr);
 #pragma unroll
     for (int fp = 0; fp < kFragRows / 2; ++fp) {
         unsigned m = 0;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int fi = fp * 2 + h;
+            if (rowHit[fi] != 0ull) {
 #pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj) {
+                for (int fj = 0; fj < kFragCols; ++fj)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (kEdge) {
-                        const int q = qBase + fi * 16 + quad * 4 + r;
-                        const bool hit =
-                            (acc[fi][fj][r] >= thr || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
-                        m = (m << 1) | (hit ? 1u : 0u);
-                    } else {
-                        // two instructions per element: the sign of acc - thr (set = no hit) is shifted in
+                    for (int r = 0; r < 4; ++r)
                         m = __builtin_amdgcn_alignbit(m, __builtin_bit_cast(unsigned, acc[fi][fj][r] - thr), 31);
-                    }
-                }
+            } else {
+                m = (m << 16) | 0xffffu;
             }
         }
-        mask[fp] = kEdge ? m : ~m;
+        mask[fp] = ~m;
     }
 }
 
