@@ -238,7 +238,8 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
         return;
     }
     // some lane has a hit: rows of blocks without one (wave-wide) are skipped, the others yield their
-    // bits, two instructions per element: the sign of acc - thr (set = no hit) is shifted in
+    // bits: the sign of acc - thr (set = no hit) is shifted in; the maximum with -inf turns a NaN
+    // (points with infinite coordinates) into "no hit", as every comparison with NaN is false
     unsigned long long rowHit[kFragRows];
 #pragma unroll
     for (int fi = 0; fi < kFragRows; ++fi) rowHit[fi] = __builtin_amdgcn_ballot_w64(rowBest[fi] >= thr);
@@ -253,7 +254,8 @@ __device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFrag
                 for (int fj = 0; fj < kFragCols; ++fj)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        m = __builtin_amdgcn_alignbit(m, __builtin_bit_cast(unsigned, acc[fi][fj][r] - thr), 31);
+                        m = __builtin_amdgcn_alignbit(
+                            m, __builtin_bit_cast(unsigned, __builtin_fmaxf(acc[fi][fj][r], -__builtin_inff()) - thr), 31);
             } else {
                 m = (m << 16) | 0xffffu;
             }

@@ -322,3 +322,21 @@ def test_caller_stream_and_repeatability(fasted):
     assert st.pairsFound == st_want.pairsFound
     for got in runs:
         assert np.array_equal(got, want)
+
+
+def test_points_with_infinite_coordinates_pair_with_nothing_but_themselves(fasted):
+    """Values beyond the FP16 range quantise to infinity (source/DataLoader/PointListBuilder.hpp:57-73); the
+    distances of such a point are NaN or infinite, every comparison with them is false
+    (source/warpMma.cuh:257), so it has no neighbours; only its self pair is reported (forced here)."""
+    n, d = 1200, 64
+    bits = datasets.uniform_bytes(n, d, seed=123)
+    eps = datasets.epsilon_for_neighbours(bits, 25)
+    odd = [5, 300, 777, 1199]
+    spoiled = bits.copy()
+    for k, i in enumerate(odd):
+        spoiled[i, (7 * k) % d] = 0x7C00 if k % 2 == 0 else 0xFC00  # +inf / -inf
+    got, st, _ = device_join(fasted, spoiled, eps)
+    clean, _, _ = device_join(fasted, bits, eps)
+    keep = ~(np.isin(clean[:, 0], odd) | np.isin(clean[:, 1], odd))
+    want = oracle.sort_pairs(np.vstack([clean[keep], [[i, i] for i in odd]]).astype(np.int32))
+    assert np.array_equal(got, want)
