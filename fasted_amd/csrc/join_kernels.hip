@@ -126,13 +126,16 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         int c = sub;
         for (; c + 3 * lanesPerRow < chunksPerRow; c += 4 * lanesPerRow) {
-            const u32x4 v0 = p[c], v1 = p[c + lanesPerRow], v2 = p[c + 2 * lanesPerRow], v3 = p[c + 3 * lanesPerRow];
+            // streaming loads: every byte is read once, nothing should displace other lines in the caches
+            const u32x4 v0 = __builtin_nontemporal_load(p + c), v1 = __builtin_nontemporal_load(p + c + lanesPerRow),
+                        v2 = __builtin_nontemporal_load(p + c + 2 * lanesPerRow),
+                        v3 = __builtin_nontemporal_load(p + c + 3 * lanesPerRow);
             part[0] = square_add(v0, part[0]);
             part[1] = square_add(v1, part[1]);
             part[2] = square_add(v2, part[2]);
             part[3] = square_add(v3, part[3]);
         }
-        for (; c < chunksPerRow; c += lanesPerRow) part[0] = square_add(p[c], part[0]);
+        for (; c < chunksPerRow; c += lanesPerRow) part[0] = square_add(__builtin_nontemporal_load(p + c), part[0]);
         acc = (part[0] + part[1]) + (part[2] + part[3]);
     }
     for (int off = lanesPerRow >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
