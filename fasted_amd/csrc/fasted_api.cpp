@@ -17,6 +17,7 @@
 #include <fstream>
 #include <iostream>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/fasted.h"
@@ -380,17 +381,62 @@ bool save_distances() {
     return v && *v && *v != '0';
 }
 
+// Decimal digits of a non-negative int, written backwards from `end`; returns the first character.
+char* write_index(char* end, int value) {
+    unsigned v = static_cast<unsigned>(value);
+    do {
+        *--end = static_cast<char>('0' + v % 10u);
+        v /= 10u;
+    } while (v);
+    return end;
+}
+
+// "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54; with distances
+// "q, c, dist\n", the three-column form results/scripts/neighbor_tables.py:102-115 also reads.
+// The lines are formatted by several threads, a slice of the list each, into buffers that are then
+// written in order (one formatted-print call per pair made large lists take minutes).
 void write_pairs_text(const std::string& path, const std::vector<FastedPair>& pairs, const std::vector<float>& dist) {
     std::FILE* f = std::fopen(path.c_str(), "w");
     if (!f) throw std::ios_base::failure("Failed to open output file: " + path);
-    // "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54; with distances
-    // "q, c, dist\n", the three-column form results/scripts/neighbor_tables.py:102-115 also reads
-    if (dist.size() == pairs.size() && !pairs.empty())
-        for (size_t i = 0; i < pairs.size(); ++i)
-            std::fprintf(f, "%d, %d, %.7g\n", pairs[i].QueryPoint, pairs[i].CandidatePoint, dist[i]);
-    else
-        for (const FastedPair& p : pairs) std::fprintf(f, "%d, %d\n", p.QueryPoint, p.CandidatePoint);
-    std::fclose(f);
+    const bool withDistance = dist.size() == pairs.size() && !pairs.empty();
+    const size_t chunk = 1u << 20;  // pairs per buffer
+    const unsigned threads = std::max(1u, std::min(fasted::host_threads("FASTED_CSV_THREADS"),
+                                                   static_cast<unsigned>((pairs.size() + chunk - 1) / chunk)));
+    std::vector<std::string> text(threads);
+    bool failed = false;
+    for (size_t base = 0; base < pairs.size() && !failed; base += chunk * threads) {
+        auto format = [&](unsigned w) {
+            const size_t lo = std::min(pairs.size(), base + w * chunk), hi = std::min(pairs.size(), lo + chunk);
+            std::string& out = text[w];
+            out.clear();
+            out.reserve((hi - lo) * (withDistance ? 40 : 24));
+            char line[64];
+            for (size_t i = lo; i < hi; ++i) {
+                char* end = line + sizeof line;
+                *--end = '\n';
+                if (withDistance) {
+                    char number[32];
+                    const int len = std::snprintf(number, sizeof number, "%.7g", dist[i]);
+                    end -= len;
+                    std::memcpy(end, number, static_cast<size_t>(len));
+                    *--end = ' ';
+                    *--end = ',';
+                }
+                end = write_index(end, pairs[i].CandidatePoint);
+                *--end = ' ';
+                *--end = ',';
+                end = write_index(end, pairs[i].QueryPoint);
+                out.append(end, static_cast<size_t>(line + sizeof line - end));
+            }
+        };
+        std::vector<std::thread> pool;
+        for (unsigned w = 1; w < threads; ++w) pool.emplace_back(format, w);
+        format(0);
+        for (auto& t : pool) t.join();
+        for (unsigned w = 0; w < threads && !failed; ++w)
+            if (!text[w].empty() && std::fwrite(text[w].data(), 1, text[w].size(), f) != text[w].size()) failed = true;
+    }
+    if (std::fclose(f) != 0 || failed) throw std::ios_base::failure("Failed to write output file: " + path);
 }
 
 Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, const std::string& datasetName) {
@@ -487,9 +533,7 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
 // built dataset that becomes the resident one; without it the resident dataset is reused (reRun).
 Results run_resident(fasted::PointTable* fresh, double epsilon, bool savePairs) {
     try {
-        std::string name;
         if (fresh) {
-            name = fresh->name;
             g_res.table = std::move(*fresh);
             g_res.uploaded = false;
             if (!quiet()) {
@@ -503,7 +547,9 @@ Results run_resident(fasted::PointTable* fresh, double epsilon, bool savePairs) 
                       << std::endl;
             std::cout << "Input Search Dimensions:\nM: " << tb.n << "\nN: " << tb.n << "\nK: " << tb.d << std::endl;
         }
-        return find_pairs_resident(epsilon, savePairs, fresh == nullptr, name);
+        // the output file of a reRun keeps the dataset's name (the reference names it "_<epsilon>.pairs":
+        // source/main.cu:203-211 clears the name there, with a note that this is not right)
+        return find_pairs_resident(epsilon, savePairs, fresh == nullptr, tb.name);
     } catch (const std::exception& e) {
         std::cout << "Error: Failed to run. " << e.what() << std::endl;
         std::exit(EXIT_FAILURE);

@@ -59,6 +59,10 @@ def test_run_from_file_saves_sorted_pairs_text(lib, tmp_path):
     r2 = lib.reRun(eps * 1.1, False)
     assert r2.pairsFound > r.pairsFound
     assert len(list(tmp_path.glob("*.pairs"))) == 1
+    # reRun with saving: the file keeps the dataset's name
+    r3 = lib.reRun(eps * 1.1, True)
+    again = tmp_path / ("points900_%f.pairs" % (eps * 1.1))
+    assert again.exists() and len(again.read_text().splitlines()) == r3.pairsStored == r2.pairsStored
     lib.releaseResources()
     lib.fasted_set_output_dir(b"")
 
