@@ -13,6 +13,7 @@ from .find_pairs import (  # noqa: F401
     compute_selectivity,
     count_pairs,
     find_epsilon,
+    find_epsilon_sampled,
     join_device,
     library_path,
     load_findpairs,
@@ -26,6 +27,6 @@ from .find_pairs import (  # noqa: F401
 )
 
 __all__ = [
-    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "join_device", "library_path",
+    "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "find_epsilon_sampled", "join_device", "library_path",
     "load_findpairs", "mmaShape", "pair_distances_device", "resident_points", "self_join", "self_join_blocked", "self_join_device", "sum_squared_device",
 ]

@@ -360,9 +360,13 @@ struct Resident {
     fasted::PointTable table;
     void* dPoints = nullptr;
     bool uploaded = false;
+    void* dSample = nullptr;  // every (n / sampleRows)-th point, for the sampled epsilon search
+    int sampleRows = 0;
     void drop_device() {
         if (dPoints) (void)hipFree(dPoints);
-        dPoints = nullptr;
+        if (dSample) (void)hipFree(dSample);
+        dPoints = dSample = nullptr;
+        sampleRows = 0;
         uploaded = false;
     }
 } g_res;
@@ -592,10 +596,68 @@ FastedJoinStats count_resident(double epsilon) {
     return st;
 }
 
+// Count-only join of an evenly spaced sample of the resident points against all of them.  Every sampled
+// point meets itself among the candidates, so found - sampleRows estimates sampleRows x selectivity.
+FastedJoinStats count_resident_sampled(double epsilon, int sampleRows) {
+    ensure_resident_uploaded();
+    const fasted::PointTable& tb = g_res.table;
+    if (sampleRows < 1) throw std::invalid_argument("sample size must be at least 1 point");
+    sampleRows = std::min(sampleRows, tb.n);
+    if (!g_res.dSample || g_res.sampleRows != sampleRows) {
+        if (g_res.dSample) (void)hipFree(g_res.dSample);
+        g_res.dSample = nullptr;
+        g_res.sampleRows = 0;
+        const size_t pitch = (size_t)tb.dPad * 2;
+        const size_t stride = (size_t)(tb.n / sampleRows);
+        HIP_CHECK(hipMalloc(&g_res.dSample, (size_t)sampleRows * pitch));
+        HIP_CHECK(hipMemcpy2D(g_res.dSample, pitch, g_res.dPoints, pitch * stride, pitch, (size_t)sampleRows,
+                              hipMemcpyDeviceToDevice));
+        g_res.sampleRows = sampleRows;
+    }
+    FastedJoinStats st{};
+    const PointSet sample{g_res.dSample, sampleRows, tb.dPad, nullptr};
+    const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
+    join_on_device(sample, all, false, tb.dPad, epsilon, nullptr, 0, 0, nullptr, &st);
+    return st;
+}
+
 double selectivity_of(unsigned long long pairsFound, int n) {
     // (|R| - |D|) / |D|, never negative (results/scripts/experiment/find_pairs.py:9-21)
     const double r = (double)pairsFound - (double)n;
     return (r > 0 ? r : 0.0) / (double)n;
+}
+
+// Epsilon for a target selectivity by the reference's procedure (results/scripts/experiment/
+// experiments.py:153-281): double epsilon (0 -> 2) until the target is reached, then half steps until the
+// selectivity is within 1 % of the target.  `probe` maps epsilon to a selectivity.
+template <typename Probe>
+double search_epsilon(double targetSelectivity, double initialEpsilon, double* selectivity, Probe&& probe) {
+    if (!(targetSelectivity > 0.0)) throw std::invalid_argument("target selectivity must be positive");
+    if (initialEpsilon < 0.0) throw std::invalid_argument("initial epsilon must not be negative");
+    const double maxEpsilon = 100000.0;
+    double lower = initialEpsilon, upper = initialEpsilon, current = 0.0;
+    while (current < targetSelectivity) {
+        lower = upper;
+        upper = (lower == 0.0) ? 2.0 : lower * 2.0;
+        if (upper > maxEpsilon)
+            throw std::runtime_error("Epsilon of " + std::to_string(upper) + " exceed the maximum value of " +
+                                     std::to_string(maxEpsilon) + ". Giving up trying to find the upper bound.");
+        current = probe(upper);
+    }
+    double eps = (upper - lower) / 2.0 + lower, last = upper;
+    current = probe(eps);
+    int guard = 0;
+    while (!(std::fabs(current - targetSelectivity) / targetSelectivity < 0.01)) {
+        const double step = std::fabs(eps - last);
+        const double next = current > targetSelectivity ? eps - 0.5 * step : eps + 0.5 * step;
+        last = eps;
+        eps = next;
+        if (++guard > 200 || next == last)  // the reference would loop forever on a plateau
+            throw std::runtime_error("epsilon search did not converge to within 1% of the target selectivity");
+        current = probe(eps);
+    }
+    if (selectivity) *selectivity = current;
+    return eps;
 }
 
 template <typename F>
@@ -756,40 +818,42 @@ int fasted_count_pairs(double epsilon, unsigned long long* pairsFound, double* k
 int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
                         int* probes) {
     return guarded([&] {
-        if (!(targetSelectivity > 0.0)) throw std::invalid_argument("target selectivity must be positive");
-        if (initialEpsilon < 0.0) throw std::invalid_argument("initial epsilon must not be negative");
         const int n = g_res.table.n;
         int count = 0;
-        auto probe = [&](double eps) {
+        const double eps = search_epsilon(targetSelectivity, initialEpsilon, selectivity, [&](double e) {
             ++count;
-            return selectivity_of(count_resident(eps).pairsFound, n);
-        };
-        // bound: double epsilon (0 -> 2) until the target is reached (experiments.py:153-195)
-        const double maxEpsilon = 100000.0;
-        double lower = initialEpsilon, upper = initialEpsilon, current = 0.0;
-        while (current < targetSelectivity) {
-            lower = upper;
-            upper = (lower == 0.0) ? 2.0 : lower * 2.0;
-            if (upper > maxEpsilon)
-                throw std::runtime_error("Epsilon of " + std::to_string(upper) + " exceed the maximum value of " +
-                                         std::to_string(maxEpsilon) + ". Giving up trying to find the upper bound.");
-            current = probe(upper);
-        }
-        // bisect by half steps until within 1 % of the target (experiments.py:198-281)
-        double eps = (upper - lower) / 2.0 + lower, last = upper;
-        current = probe(eps);
-        int guard = 0;
-        while (!(std::fabs(current - targetSelectivity) / targetSelectivity < 0.01)) {
-            const double step = std::fabs(eps - last);
-            const double next = current > targetSelectivity ? eps - 0.5 * step : eps + 0.5 * step;
-            last = eps;
-            eps = next;
-            if (++guard > 200 || next == last)  // the reference would loop forever on a plateau
-                throw std::runtime_error("epsilon search did not converge to within 1% of the target selectivity");
-            current = probe(eps);
-        }
+            return selectivity_of(count_resident(e).pairsFound, n);
+        });
         if (epsilon) *epsilon = eps;
-        if (selectivity) *selectivity = current;
+        if (probes) *probes = count;
+    });
+}
+
+int fasted_count_pairs_sampled(double epsilon, int sample_rows, unsigned long long* pairsFound, int* sampledRows,
+                               double* kernelSeconds) {
+    return guarded([&] {
+        const FastedJoinStats st = count_resident_sampled(epsilon, sample_rows);
+        if (pairsFound) *pairsFound = st.pairsFound;
+        if (sampledRows) *sampledRows = g_res.sampleRows;
+        if (kernelSeconds) *kernelSeconds = (st.sumSquaredMs + st.joinMs) / 1000.0;
+    });
+}
+
+int fasted_find_epsilon_sampled(double targetSelectivity, double initialEpsilon, int sample_rows, double* epsilon,
+                                double* selectivity, int* probes) {
+    return guarded([&] {
+        int count = 0;
+        double estimate = 0.0;
+        const double eps = search_epsilon(targetSelectivity, initialEpsilon, &estimate, [&](double e) {
+            ++count;
+            const FastedJoinStats st = count_resident_sampled(e, sample_rows);
+            return selectivity_of(st.pairsFound, g_res.sampleRows);
+        });
+        // one full count at the end: the selectivity reported is the dataset's, not the sample's
+        ++count;
+        const double full = selectivity_of(count_resident(eps).pairsFound, g_res.table.n);
+        if (epsilon) *epsilon = eps;
+        if (selectivity) *selectivity = full;
         if (probes) *probes = count;
     });
 }

@@ -126,6 +126,12 @@ def load_findpairs(path: str = None):
                                                  c.c_void_p]
     lib.fasted_set_save_distances.restype = None
     lib.fasted_set_save_distances.argtypes = [c.c_int]
+    lib.fasted_count_pairs_sampled.restype = c.c_int
+    lib.fasted_count_pairs_sampled.argtypes = [c.c_double, c.c_int, c.POINTER(c.c_ulonglong), c.POINTER(c.c_int),
+                                               c.POINTER(c.c_double)]
+    lib.fasted_find_epsilon_sampled.restype = c.c_int
+    lib.fasted_find_epsilon_sampled.argtypes = [c.c_double, c.c_double, c.c_int, c.POINTER(c.c_double),
+                                                c.POINTER(c.c_double), c.POINTER(c.c_int)]
     lib.fasted_sum_squared_device.restype = c.c_int
     lib.fasted_sum_squared_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_void_p, c.c_void_p]
     lib.fasted_raster_coord.restype = c.c_int
@@ -245,6 +251,16 @@ def find_epsilon(target_selectivity, initial_epsilon=0.0):
     eps, sel, probes = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
     _check(lib, lib.fasted_find_epsilon(float(target_selectivity), float(initial_epsilon), ctypes.byref(eps),
                                         ctypes.byref(sel), ctypes.byref(probes)))
+    return eps.value, sel.value, probes.value
+
+
+def find_epsilon_sampled(target_selectivity, sample_rows=16384, initial_epsilon=0.0):
+    """find_epsilon on sampled probes (sample_rows/N of the work each) plus one full count at the end:
+    (epsilon, selectivity of the whole dataset, probes)."""
+    lib = load_findpairs()
+    eps, sel, probes = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
+    _check(lib, lib.fasted_find_epsilon_sampled(float(target_selectivity), float(initial_epsilon), int(sample_rows),
+                                                ctypes.byref(eps), ctypes.byref(sel), ctypes.byref(probes)))
     return eps.value, sel.value, probes.value
 
 

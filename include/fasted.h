@@ -186,6 +186,17 @@ int fasted_count_pairs(double epsilon, unsigned long long* pairsFound, double* k
 int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
                         int* probes);
 
+/* The same probe and the same search on an evenly spaced sample of `sample_rows` query points against all
+ * points (sample_rows/N of the work per probe): *pairsFound - *sampledRows estimates sampledRows x
+ * selectivity.  fasted_find_epsilon_sampled runs the search of fasted_find_epsilon on sampled probes and
+ * ends with one full count, so *selectivity is the dataset's; it can miss the 1 % window by the sampling
+ * error (about 1/sqrt(sample_rows x selectivity)).  The reference pays a full run per probe
+ * (results/scripts/experiment/experiments.py:228-281 via find_pairs). */
+int fasted_count_pairs_sampled(double epsilon, int sample_rows, unsigned long long* pairsFound, int* sampledRows,
+                               double* kernelSeconds);
+int fasted_find_epsilon_sampled(double targetSelectivity, double initialEpsilon, int sample_rows, double* epsilon,
+                                double* selectivity, int* probes);
+
 /* Resident dataset: padded FP16 bit patterns (host copy) and its name
  * (PointGenerator::getName, source/DataLoader/PointGenerator.hpp:27-30). */
 const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad);

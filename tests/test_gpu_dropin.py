@@ -119,6 +119,31 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     lib.releaseResources()
 
 
+def test_sampled_epsilon_search(lib):
+    """The search on sampled probes: the sampled count equals the count of the same rows in the full pair
+    list, and the epsilon found lands close to the full search's at a fraction of the work."""
+    import ctypes
+
+    import fasted_amd
+    from fasted_amd import experiments as ex
+
+    n, d = 20000, 64
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    eps_full, sel_full, probes_full = fasted_amd.find_epsilon(30.0)
+    eps_s, sel_s, probes_s = fasted_amd.find_epsilon_sampled(30.0, sample_rows=2000)
+    assert probes_s >= 4 and abs(eps_s - eps_full) / eps_full < 0.01
+    assert ex.within_percent(sel_s, 30.0, 0.05)  # the dataset's selectivity at the sampled search's epsilon
+    # the sampled probe counts exactly the pairs whose query point is one of the sampled rows
+    found, rows, secs = ctypes.c_ulonglong(), ctypes.c_int(), ctypes.c_double()
+    assert lib.fasted_count_pairs_sampled(eps_s, 2000, ctypes.byref(found), ctypes.byref(rows), ctypes.byref(secs)) == 0
+    assert rows.value == 2000
+    bits, _, _, _ = fasted_amd.resident_points()
+    pairs, total = fasted_amd.self_join(bits[:n, :d].copy(), eps_s)
+    sampled_rows = np.arange(2000) * (n // 2000)
+    assert found.value == int(np.isin(pairs[:, 0], sampled_rows).sum())
+    lib.releaseResources()
+
+
 def test_experiment_sweep_reproduces_the_reference_result_records(lib, tmp_path):
     """The size x dimensionality sweep of the reference's experiment driver, run on the library: for
     the shapes small enough to run here the records of results/speed_results/
