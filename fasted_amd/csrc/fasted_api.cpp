@@ -860,8 +860,15 @@ int fasted_find_epsilon_sampled(double targetSelectivity, double initialEpsilon,
 
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col) {
     if (n < 1 || !row || !col) return 0;
-    return fasted::raster_coord(idx, n, n, row, col);
+    return fasted::raster_coord(idx, n, n, false, row, col);
 }
+
+int fasted_raster_coord_symmetric(unsigned long long idx, long long n, int* row, int* col) {
+    if (n < 1 || !row || !col) return 0;
+    return fasted::raster_coord(idx, n, n, true, row, col);
+}
+
+unsigned long long fasted_raster_count_symmetric(long long n) { return n < 1 ? 0ull : fasted::raster_count(n, n, true); }
 
 int fasted_lds_chunk_slot(int row, int chunk) { return fasted::lds_chunk_slot(row, chunk); }
 

@@ -28,8 +28,9 @@ struct JoinLaunch {
 };
 
 // Host mirror of the device tile order.
-unsigned long long raster_count(long long nQ, long long nC);
-int raster_coord(unsigned long long idx, long long nQ, long long nC, int* row, int* col);
+// upperOnly: the order of a symmetric self-join (super-squares on and above the diagonal only).
+unsigned long long raster_count(long long nQ, long long nC, bool upperOnly = false);
+int raster_coord(unsigned long long idx, long long nQ, long long nC, bool upperOnly, int* row, int* col);
 int counter_words();
 unsigned long long tile_count(long long nQ, long long nC);  // 256x256 tiles the kernel processes
 // Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).

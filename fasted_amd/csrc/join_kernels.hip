@@ -69,6 +69,7 @@ __host__ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 struct Raster {
     unsigned tileRows, tileCols;      // 256-point tiles along the queries / the candidates
     unsigned squareCols;              // super-squares per row of super-squares
+    unsigned upperOnly;               // symmetric self-join: only the super-squares on and above the diagonal
     unsigned long long perQueue;  // pops each queue serves
 };
 
@@ -80,13 +81,16 @@ constexpr int kCounterFound = 0;
 constexpr int kQueueBase = 16, kQueueStride = 16;  // queue heads sit on separate 128-byte lines
 constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
-__host__ __device__ inline Raster make_raster(long long nQueries, long long nCandidates) {
+__host__ __device__ inline Raster make_raster(long long nQueries, long long nCandidates, bool upperOnly = false) {
     Raster r;
     r.tileRows = (unsigned)((nQueries + kTile - 1) / kTile);
     r.tileCols = (unsigned)((nCandidates + kTile - 1) / kTile);
     const unsigned squareRows = (r.tileRows + kRaster - 1) / kRaster;
     r.squareCols = (r.tileCols + kRaster - 1) / kRaster;
-    r.perQueue = (unsigned long long)squareRows * r.squareCols * kSubTiles;
+    r.upperOnly = (upperOnly && squareRows == r.squareCols) ? 1u : 0u;
+    const unsigned long long squares = r.upperOnly ? (unsigned long long)squareRows * (squareRows + 1) / 2
+                                                   : (unsigned long long)squareRows * r.squareCols;
+    r.perQueue = squares * kSubTiles;
     return r;
 }
 
@@ -96,8 +100,25 @@ __host__ __device__ inline void raster_decode(const Raster& r, unsigned q, unsig
                                               unsigned* tc) {
     const unsigned long long sq = t / kSubTiles;
     const unsigned local = (unsigned)(t % kSubTiles);
-    *tr = (unsigned)(sq / r.squareCols) * kRaster + (q >> 1) * kSubRows + local / kSubCols;
-    *tc = (unsigned)(sq % r.squareCols) * kRaster + (q & 1) * kSubCols + local % kSubCols;
+    unsigned squareRow, squareCol;
+    if (r.upperOnly) {
+        // row-major over the upper triangle: row i starts at i*S - i*(i-1)/2; estimate, then correct
+        const unsigned long long S = r.squareCols;
+        const double b = 2.0 * (double)S + 1.0;
+        long long i = (long long)((b - __builtin_sqrt(b * b - 8.0 * (double)sq)) * 0.5);
+        if (i < 0) i = 0;
+        if (i >= (long long)S) i = (long long)S - 1;
+        auto start = [S](long long row) { return (unsigned long long)row * S - (unsigned long long)(row * (row - 1) / 2); };
+        while (i > 0 && start(i) > sq) --i;
+        while (i + 1 < (long long)S && start(i + 1) <= sq) ++i;
+        squareRow = (unsigned)i;
+        squareCol = (unsigned)(i + (long long)(sq - start(i)));
+    } else {
+        squareRow = (unsigned)(sq / r.squareCols);
+        squareCol = (unsigned)(sq % r.squareCols);
+    }
+    *tr = squareRow * kRaster + (q >> 1) * kSubRows + local / kSubCols;
+    *tc = squareCol * kRaster + (q & 1) * kSubCols + local % kSubCols;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -638,19 +659,22 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
 }  // namespace
 
-unsigned long long raster_count(long long nQ, long long nC) { return make_raster(nQ, nC).perQueue * kQueues; }
+unsigned long long raster_count(long long nQ, long long nC, bool upperOnly) {
+    return make_raster(nQ, nC, upperOnly).perQueue * kQueues;
+}
 
 // Index idx enumerates the queues round-robin: queue idx % 8, position idx / 8 -- the order in
 // which eight equally fast XCDs would take the tiles.  Returns 0 past the end, 2 for a padding
 // tile that the kernel skips, 1 for a real tile.
-int raster_coord(unsigned long long idx, long long nQ, long long nC, int* row, int* col) {
-    const Raster r = make_raster(nQ, nC);
+// With upperOnly (symmetric self-join) the tiles below the diagonal count as skipped as well.
+int raster_coord(unsigned long long idx, long long nQ, long long nC, bool upperOnly, int* row, int* col) {
+    const Raster r = make_raster(nQ, nC, upperOnly);
     if (idx >= r.perQueue * kQueues) return 0;
     unsigned tr, tc;
     raster_decode(r, (unsigned)(idx % kQueues), idx / kQueues, &tr, &tc);
     *row = (int)tr * kTile;
     *col = (int)tc * kTile;
-    return (tr < r.tileRows && tc < r.tileCols) ? 1 : 2;
+    return (tr < r.tileRows && tc < r.tileCols && !(upperOnly && tc < tr)) ? 1 : 2;
 }
 
 int counter_words() { return kCounterWords; }
@@ -717,7 +741,7 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
     p.counters = l.counters;
     p.pairs = static_cast<int2*>(l.pairs);
     p.cap = l.cap;
-    p.raster = make_raster(l.nQ, l.nC);
+    p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0);
     unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
     unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;

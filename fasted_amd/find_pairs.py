@@ -138,6 +138,10 @@ def load_findpairs(path: str = None):
     lib.fasted_raster_coord.argtypes = [c.c_ulonglong, c.c_longlong, c.POINTER(c.c_int), c.POINTER(c.c_int)]
     lib.fasted_raster_count.restype = c.c_ulonglong
     lib.fasted_raster_count.argtypes = [c.c_longlong]
+    lib.fasted_raster_coord_symmetric.restype = c.c_int
+    lib.fasted_raster_coord_symmetric.argtypes = [c.c_ulonglong, c.c_longlong, c.POINTER(c.c_int), c.POINTER(c.c_int)]
+    lib.fasted_raster_count_symmetric.restype = c.c_ulonglong
+    lib.fasted_raster_count_symmetric.argtypes = [c.c_longlong]
     lib.fasted_load_exponential_dataset.restype = c.c_int
     lib.fasted_load_exponential_dataset.argtypes = [c.c_int, c.c_int, c.c_double, c.c_double]
     lib.fasted_load_file.restype = c.c_int

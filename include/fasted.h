@@ -157,6 +157,12 @@ int fasted_sum_squared_device(const void* d_points, long long n, int d, long lon
  * (source/rasterizer/onDemandRasterizer.cuh:78-108). */
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col);
 unsigned long long fasted_raster_count(long long n);
+/* The same for a FASTED_SYMMETRIC join: only the 16x16-tile squares on and above the diagonal are
+ * enumerated (row-major over the upper triangle), and tiles below the diagonal inside the diagonal squares
+ * return 2 like padding tiles.  No counterpart in the reference, which always walks the full grid
+ * (source/rasterizer/onDemandRasterizer.cuh:50-71). */
+int fasted_raster_coord_symmetric(unsigned long long idx, long long n, int* row, int* col);
+unsigned long long fasted_raster_count_symmetric(long long n);
 
 /* LDS placement of the kernel's operand tiles: the 16-byte chunk `chunk` (0..7) of row `row` of a
  * 64-wide k-slab is stored at the returned slot (0..7) of that row's 128 bytes.  Host mirror of the

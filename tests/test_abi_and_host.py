@@ -178,6 +178,26 @@ def test_tile_queues_cover_every_tile_exactly_once(lib, n):
     assert lib.fasted_raster_coord(total, n, ctypes.byref(row), ctypes.byref(col)) == 0
 
 
+@pytest.mark.parametrize("n", [1, 256, 4097, 5000, 70_000, 150_000])
+def test_symmetric_tile_queues_cover_the_upper_triangle_exactly_once(lib, n):
+    """The order of a FASTED_SYMMETRIC join: every tile on or above the diagonal exactly once, nothing
+    else marked as work, and about half as many queue positions as the full order."""
+    total = lib.fasted_raster_count_symmetric(n)
+    tiles = -(-n // 256)
+    seen = np.zeros((tiles, tiles), dtype=np.int32)
+    row, col = ctypes.c_int(), ctypes.c_int()
+    for idx in range(total):
+        kind = lib.fasted_raster_coord_symmetric(idx, n, ctypes.byref(row), ctypes.byref(col))
+        assert kind in (1, 2)
+        if kind == 1:
+            assert row.value <= col.value
+            seen[row.value // 256, col.value // 256] += 1
+    assert lib.fasted_raster_coord_symmetric(total, n, ctypes.byref(row), ctypes.byref(col)) == 0
+    assert np.array_equal(seen, np.triu(np.ones((tiles, tiles), dtype=np.int32)))
+    squares = -(-tiles // 16)
+    assert total == 256 * squares * (squares + 1) // 2 <= lib.fasted_raster_count(n)
+
+
 def test_tile_queue_locality(lib):
     """32 consecutive positions of one queue are one 4 x 8 block of tiles (one XCD's share of a
     16 x 16 super-square), and the 8 queues together tile that super-square."""
