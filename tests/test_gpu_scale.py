@@ -103,9 +103,9 @@ def test_config4_clustered_500k_x_960(env):
 
 
 def test_config5_output_heavy_2m_x_384(env):
-    st = run_config(env, "c5", sample_rows=1024)
+    st = run_config(env, "c5", sample_rows=1024, oracle_rows=4)
     assert st.pairsFound > 2e8  # the output-heavy case really is output heavy
 
 
 def test_config3_headline_1m_x_4096(env):
-    run_config(env, "c3", sample_rows=1024)
+    run_config(env, "c3", sample_rows=1024, oracle_rows=4)

@@ -227,6 +227,38 @@ def _five():
     return np.array([[1, 1], [2, 2], [3, 3], [4, 4], [5, 5]], dtype=np.int32)
 
 
+def test_pair_distances_f64_against_numpy_and_closed_forms():
+    """The distances the epsilon-band classifier judges disagreements by: the sum of squared differences in
+    FP64 (exact on FP16 inputs up to FP64 rounding), against numpy on random pairs, and on pairs whose
+    distance is known in closed form (a point with itself; unit vectors; a 3-4-5 triangle).  A swapped
+    index, a missed square root or a distance formed from the expansion s_q + s_c - 2 q.c (which cancels)
+    fails one of them."""
+    rng = np.random.default_rng(21)
+    n, d = 300, 77  # odd dimensionality: no padding column may be touched
+    x = (rng.standard_normal((n, d)) * 3.0).astype(np.float16)
+    bits = x.view(np.uint16)
+    pairs = rng.integers(0, n, size=(5000, 2)).astype(np.int32)
+    got = oracle.pair_distances_f64(bits, pairs)
+    x64 = x.astype(np.float64)
+    want = np.sqrt(((x64[pairs[:, 0]] - x64[pairs[:, 1]]) ** 2).sum(1))
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got, want, rtol=1e-14, atol=0.0)
+    # not symmetric inputs by accident: (q, c) and (c, q) give the same distance, but different pairs do not
+    np.testing.assert_array_equal(got, oracle.pair_distances_f64(bits, pairs[:, ::-1]))
+    assert len(np.unique(got)) > 4000
+
+    fix = np.zeros((5, 8), dtype=np.float16)
+    fix[1, 0] = 1.0
+    fix[2, 1] = 1.0
+    fix[3, 0], fix[3, 1] = 3.0, 4.0
+    fix[4] = 1000.0  # large norm: the expansion would lose the small difference to fix[4] itself
+    fb = fix.view(np.uint16)
+    closed = oracle.pair_distances_f64(fb, [(0, 0), (4, 4), (0, 1), (1, 2), (0, 3), (3, 0), (1, 3)])
+    np.testing.assert_array_equal(closed[:2], [0.0, 0.0])
+    np.testing.assert_allclose(closed[2:], [1.0, np.sqrt(2.0), 5.0, 5.0, np.sqrt(4.0 + 16.0)], rtol=1e-15)
+    assert oracle.pair_distances_f64(fb, np.zeros((0, 2), dtype=np.int32)).shape == (0,)
+
+
 @pytest.mark.parametrize("delete,side,expect", [
     # the cases of results/scripts/test_accuracy.py: (both, right_only, left_only, left_total, right_total)
     (None, None, (5, 0, 0, 5, 5)),
