@@ -23,10 +23,11 @@ from .find_pairs import (  # noqa: F401
     self_join,
     self_join_blocked,
     self_join_device,
+    self_join_device_noalloc,
     sum_squared_device,
 )
 
 __all__ = [
     "FastedJoinStats", "FastedPair", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "find_epsilon_sampled", "join_device", "library_path",
-    "load_findpairs", "mmaShape", "pair_distances_device", "resident_points", "self_join", "self_join_blocked", "self_join_device", "sum_squared_device",
+    "load_findpairs", "mmaShape", "pair_distances_device", "resident_points", "self_join", "self_join_blocked", "self_join_device", "self_join_device_noalloc", "sum_squared_device",
 ]

@@ -80,12 +80,62 @@ struct Workspace {
     }
 } g_ws;
 
-struct EventTimer {
-    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
-    EventTimer() {
-        for (auto& e : ev) HIP_CHECK(hipEventCreate(&e));
+// ---- the entry point that allocates nothing --------------------------------------------------
+// Its kernels use the same two pieces of device memory beyond inputs and outputs as every other join here:
+// the counter block (pair counter + queue heads) and the squared norms.  They live in one file-scope device
+// array instead of hipMalloc'ed memory; each GPU the library runs on holds its own copy at its own address,
+// looked up once per device.  Host code never uses the array's name as an address: only `base`.
+constexpr size_t kNoAllocMaxPoints = (size_t)1 << 22;  // 4 Mi points: 16 MiB of squared norms
+constexpr size_t kNoAllocCounterBytes = 4096;          // counter block (1152 bytes used)
+constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + kNoAllocMaxPoints * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+constexpr int kMaxDevices = 64;
+struct DeviceScratch {
+    unsigned char* base = nullptr;  // device address of `scratch` on this device
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+} g_deviceScratch[kMaxDevices];
+
+// First call on the current device: looks up the device's copy of `scratch` and creates the timing
+// events.  Later calls only read the table.
+DeviceScratch& device_scratch() {
+    int dev = 0;
+    HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) throw std::invalid_argument("device index out of range");
+    DeviceScratch& ds = g_deviceScratch[dev];
+    if (!ds.base) {
+        void* ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        for (auto& e : ds.ev) HIP_CHECK(hipEventCreate(&e));
+        ds.base = static_cast<unsigned char*>(ptr);
     }
+    return ds;
+}
+
+// Where a join keeps its counters and (unless the caller brings a buffer) its squared norms, and the
+// events it times itself with.  Default: the library workspace, events created for the call.
+struct JoinScratch {
+    unsigned long long* counters;
+    float* sums;
+    hipEvent_t* ev;  // three events
+};
+
+// Three events around the two timed stages; created for the call, or borrowed from the caller.
+struct EventTimer {
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    bool owned;
+    explicit EventTimer(hipEvent_t* borrowed = nullptr) : owned(borrowed == nullptr) {
+        for (int i = 0; i < 3; ++i) {
+            if (borrowed)
+                ev[i] = borrowed[i];
+            else
+                HIP_CHECK(hipEventCreate(&ev[i]));
+        }
+    }
+    EventTimer(const EventTimer&) = delete;
+    EventTimer& operator=(const EventTimer&) = delete;
     ~EventTimer() {
+        if (!owned) return;
         for (auto& e : ev)
             if (e) (void)hipEventDestroy(e);
     }
@@ -119,18 +169,28 @@ struct PointSet {
 // queue/pair-counter reset and the join kernel; then counters come back and the stored pairs
 // are sorted outside the TFLOPS window.  `c.ptr == q.ptr` with selfJoin computes the norms once.
 void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon, void* dPairs,
-                    unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats) {
+                    unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats,
+                    const JoinScratch* fixed = nullptr) {
     validate_shape(q.n, d, q.ld);
     validate_shape(c.n, d, c.ld);
     if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
     const int dPad = round_up(d, fasted::kSlabK);
-    g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
-    float* sumsQ = q.sums ? q.sums : g_ws.sums;
-    float* sumsC = selfJoin ? sumsQ : (c.sums ? c.sums : g_ws.sums + q.n);
+    EventTimer t(fixed ? fixed->ev : nullptr);
+    unsigned long long* counters = nullptr;
+    float* wsSums = nullptr;
+    if (fixed) {
+        counters = fixed->counters;
+        wsSums = fixed->sums;
+    } else {
+        g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
+        counters = g_ws.counters;
+        wsSums = g_ws.sums;
+    }
+    float* sumsQ = q.sums ? q.sums : wsSums;
+    float* sumsC = selfJoin ? sumsQ : (c.sums ? c.sums : wsSums + q.n);
     if ((flags & FASTED_SKIP_SUMS) && (!q.sums || (!selfJoin && !c.sums)))
         throw std::invalid_argument("FASTED_SKIP_SUMS needs the squared-norm buffers");
 
-    EventTimer t;
     HIP_CHECK(hipEventRecord(t.ev[0], stream));
     if (!(flags & FASTED_SKIP_SUMS)) {
         HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, stream));
@@ -151,11 +211,11 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
     jl.sumsQ = sumsQ;
     jl.sumsC = sumsC;
-    jl.counters = g_ws.counters;
+    jl.counters = counters;
     jl.pairs = dPairs;
     jl.cap = cap;
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
-    HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, stream));
+    HIP_CHECK(fasted::launch_reset_counters(counters, false, stream));
     HIP_CHECK(fasted::launch_join(jl, stream));
     HIP_CHECK(hipEventRecord(t.ev[2], stream));
     HIP_CHECK(hipStreamSynchronize(stream));
@@ -163,7 +223,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
     // counted only (source/pair.cuh:123-133), so stored = min(found, capacity)
     unsigned long long cnt[4] = {0, 0, 0, 0};
-    HIP_CHECK(hipMemcpy(cnt, g_ws.counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);
     float sortMs = 0.f;
@@ -710,6 +770,26 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
         if (!d_points) throw std::invalid_argument("points pointer is null");
         const PointSet all{d_points, n, ld, d_sums};
         join_on_device(all, all, true, d, epsilon, d_pairs, cap, flags, static_cast<hipStream_t>(stream), stats);
+    });
+}
+
+int fasted_self_join_device_noalloc(const void* d_points, long long n, int d, long long ld, double epsilon,
+                                    FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
+                                    FastedJoinStats* stats) {
+    return guarded([&] {
+        if (!d_points) throw std::invalid_argument("points pointer is null");
+        if (n > (long long)kNoAllocMaxPoints)
+            throw std::invalid_argument("fasted_self_join_device_noalloc holds the squared norms of at most " +
+                                        std::to_string(kNoAllocMaxPoints) + " points; got " + std::to_string(n));
+        if (flags & FASTED_SORT_PAIRS)
+            throw std::invalid_argument("fasted_self_join_device_noalloc cannot sort: the sort allocates device memory");
+        if (flags & FASTED_SKIP_SUMS)
+            throw std::invalid_argument("fasted_self_join_device_noalloc computes the squared norms itself");
+        DeviceScratch& ds = device_scratch();
+        const JoinScratch js{reinterpret_cast<unsigned long long*>(ds.base),
+                             reinterpret_cast<float*>(ds.base + kNoAllocCounterBytes), ds.ev};
+        const PointSet all{d_points, n, ld, nullptr};
+        join_on_device(all, all, true, d, epsilon, d_pairs, cap, flags, static_cast<hipStream_t>(stream), stats, &js);
     });
 }
 

@@ -116,6 +116,10 @@ def load_findpairs(path: str = None):
     lib.fasted_self_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_double, c.c_void_p,
                                             c.c_void_p, c.c_ulonglong, c.c_uint, c.c_void_p,
                                             c.POINTER(FastedJoinStats)]
+    lib.fasted_self_join_device_noalloc.restype = c.c_int
+    lib.fasted_self_join_device_noalloc.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_double,
+                                                    c.c_void_p, c.c_ulonglong, c.c_uint, c.c_void_p,
+                                                    c.POINTER(FastedJoinStats)]
     lib.fasted_join_device.restype = c.c_int
     lib.fasted_join_device.argtypes = [c.c_void_p, c.c_longlong, c.c_longlong, c.c_void_p, c.c_longlong, c.c_longlong,
                                        c.c_int, c.c_double, c.c_void_p, c.c_void_p, c.c_void_p, c.c_ulonglong, c.c_uint,
@@ -217,6 +221,15 @@ def self_join_device(points_ptr, n, d, ld, epsilon, pairs_ptr, cap, sums_ptr=Non
     st = FastedJoinStats()
     _check(lib, lib.fasted_self_join_device(points_ptr, n, d, ld, float(epsilon), sums_ptr, pairs_ptr, cap, flags,
                                             stream, ctypes.byref(st)))
+    return st
+
+
+def self_join_device_noalloc(points_ptr, n, d, ld, epsilon, pairs_ptr, cap, flags=0, stream=None):
+    """self_join_device without any device allocation inside the call (pairs unsorted, n <= 4 Mi)."""
+    lib = load_findpairs()
+    st = FastedJoinStats()
+    _check(lib, lib.fasted_self_join_device_noalloc(points_ptr, n, d, ld, float(epsilon), pairs_ptr, cap, flags,
+                                                    stream, ctypes.byref(st)))
     return st
 
 

@@ -125,6 +125,19 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
                             FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
                             FastedJoinStats* stats);
 
+/* fasted_self_join_device for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The queue
+ * heads, the pair counter and the squared norms live in a device array that is part of the library image
+ * (4 KiB + 16 MiB per GPU, held until the process ends) instead of allocated workspace; the call makes no
+ * hipMalloc / hipFree and calls no allocating library routine.  Limits, each refused with an error:
+ * n <= 4 194 304 points; FASTED_SORT_PAIRS (the sort needs device buffers; the pairs come back in
+ * arbitrary order) and FASTED_SKIP_SUMS are not accepted.  Every call on one GPU shares that GPU's array:
+ * calls that overlap on one GPU race.  Same results as fasted_self_join_device otherwise; the first call on
+ * a device looks up the array's address and creates three timing events. */
+int fasted_self_join_device_noalloc(const void* d_points, long long n, int d, long long ld, double epsilon,
+                                    FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
+                                    FastedJoinStats* stats);
+
 /* Join of two different sets: every pair (q, c), q indexing the queries and c the candidates, with
  * dist <= epsilon; no pair is forced (there are no self pairs).  Same buffer rules per set as
  * fasted_self_join_device.  The reference's device parameters already carry distinct query and
