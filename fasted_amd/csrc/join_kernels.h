@@ -44,6 +44,7 @@ hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned l
                                hipStream_t stream);
 hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
 
+
 // Row-major sort of `count` stored pairs (pair_sort.hip).
 hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream);
 

@@ -28,12 +28,12 @@
 
 #include <type_traits>
 
+#include "join_device.hpp"
+#include "tile_order.hpp"
+
 namespace fasted {
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 512;                       // 8 waves: 2 (rows) x 4 (cols)
 constexpr int kRowBytes = kSlabK * 2;               // one LDS row of a slab: 128 B = 8 chunks of 16 B
@@ -50,75 +50,26 @@ static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
-// 16-byte chunk c of LDS row r lives at chunk slot c ^ swz(r).  A row is 128 B, so row parity
-// picks the half of the 64 four-byte banks and the slot picks 4 banks inside it.  gfx950 serves
-// a ds_read_b128 in four phases of 16 lanes -- {0-3,12-15,20-23,24-27}, {4-7,8-11,16-19,28-31}
-// and the same two groups +32 -- and the fragment read of v_mfma_f32_16x16x32_f16 has lane l on
-// row l%16, chunk 4*ks + l/16.  With swz(r) = (r>>1)&7 every phase touches 16 distinct
-// (parity, slot) pairs, i.e. all 64 banks once: no bank conflict (checked exhaustively on the
-// host by tests, and with the SQ_LDS_BANK_CONFLICT counter on the device).
-__host__ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+// Operand rows of the 256x256 kernel are 128 bytes (a 64-wide k-slab): see lds_swizzle128 in
+// tile_order.hpp (conflict freedom is checked exhaustively on the host by tests, and with the
+// SQ_LDS_BANK_CONFLICT counter on the device).
+__host__ __device__ __forceinline__ int swz(int row) { return lds_swizzle128(row); }
 
-// Work queues.  The N x N matrix of 256x256 tiles is cut into super-squares of 16 x 16 tiles;
-// a super-square is cut into 8 sub-rectangles of 4 x 8 tiles, one per XCD (accelerator die).
-// Each XCD has its own queue head: its t-th pop is tile (t % 32) of its sub-rectangle of
-// super-square t / 32.  The 32 workgroups resident on one XCD therefore work on 4 query panels
-// and 8 candidate panels at a time and share them through that XCD's L2, and all 8 XCDs stay
-// inside one super-square (16 + 16 panels) that the Infinity Cache holds.  An XCD whose queue
-// is exhausted steals from the next XCD's queue, so the tail stays balanced.
-struct Raster {
-    unsigned tileRows, tileCols;      // 256-point tiles along the queries / the candidates
-    unsigned squareCols;              // super-squares per row of super-squares
-    unsigned upperOnly;               // symmetric self-join: only the super-squares on and above the diagonal
-    unsigned long long perQueue;  // pops each queue serves
-};
-
-constexpr int kQueues = 8;                 // one per XCD
+// Work queues of the 256x256 kernel (tile_order.hpp): an XCD's sub-rectangle is 4 x 8 tiles, so the 32
+// workgroups resident on one XCD work on 4 query panels and 8 candidate panels at a time.  An XCD whose
+// queue is exhausted steals from the next XCD's queue, so the tail stays balanced.
+typedef TileOrder Raster;
 constexpr int kSubRows = 4, kSubCols = 8;  // sub-rectangle of one XCD inside a super-square
 constexpr int kSubTiles = kSubRows * kSubCols;
 static_assert(kRaster == 16 && kSubTiles * kQueues == kRaster * kRaster, "8 sub-rectangles tile a super-square");
-constexpr int kCounterFound = 0;
-constexpr int kQueueBase = 16, kQueueStride = 16;  // queue heads sit on separate 128-byte lines
-constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
 __host__ __device__ inline Raster make_raster(long long nQueries, long long nCandidates, bool upperOnly = false) {
-    Raster r;
-    r.tileRows = (unsigned)((nQueries + kTile - 1) / kTile);
-    r.tileCols = (unsigned)((nCandidates + kTile - 1) / kTile);
-    const unsigned squareRows = (r.tileRows + kRaster - 1) / kRaster;
-    r.squareCols = (r.tileCols + kRaster - 1) / kRaster;
-    r.upperOnly = (upperOnly && squareRows == r.squareCols) ? 1u : 0u;
-    const unsigned long long squares = r.upperOnly ? (unsigned long long)squareRows * (squareRows + 1) / 2
-                                                   : (unsigned long long)squareRows * r.squareCols;
-    r.perQueue = squares * kSubTiles;
-    return r;
+    return make_tile_order(nQueries, nCandidates, kTile, kTile, kSubRows, kSubCols, upperOnly);
 }
 
-// Pop t of queue q -> tile (row, col) in tile units.  Tiles outside the tileRows x tileCols grid are
-// padding of the last super-squares: the caller skips them.
 __host__ __device__ inline void raster_decode(const Raster& r, unsigned q, unsigned long long t, unsigned* tr,
                                               unsigned* tc) {
-    const unsigned long long sq = t / kSubTiles;
-    const unsigned local = (unsigned)(t % kSubTiles);
-    unsigned squareRow, squareCol;
-    if (r.upperOnly) {
-        // row-major over the upper triangle: row i starts at i*S - i*(i-1)/2; estimate, then correct
-        const unsigned long long S = r.squareCols;
-        const double b = 2.0 * (double)S + 1.0;
-        long long i = (long long)((b - __builtin_sqrt(b * b - 8.0 * (double)sq)) * 0.5);
-        if (i < 0) i = 0;
-        if (i >= (long long)S) i = (long long)S - 1;
-        auto start = [S](long long row) { return (unsigned long long)row * S - (unsigned long long)(row * (row - 1) / 2); };
-        while (i > 0 && start(i) > sq) --i;
-        while (i + 1 < (long long)S && start(i + 1) <= sq) ++i;
-        squareRow = (unsigned)i;
-        squareCol = (unsigned)(i + (long long)(sq - start(i)));
-    } else {
-        squareRow = (unsigned)(sq / r.squareCols);
-        squareCol = (unsigned)(sq % r.squareCols);
-    }
-    *tr = squareRow * kRaster + (q >> 1) * kSubRows + local / kSubCols;
-    *tc = squareCol * kRaster + (q & 1) * kSubCols + local % kSubCols;
+    tile_order_decode(r, kSubRows, kSubCols, q, t, tr, tc);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -183,120 +134,6 @@ __global__ void __launch_bounds__(256) offset_pairs_kernel(int2* pairs, unsigned
 }
 
 // ------------------------------------------------------------------------------------------
-struct JoinParams {
-    const u32x4* ptsQ;  // query rows
-    const u32x4* ptsC;  // candidate rows (the same buffer for a self-join)
-    long long ldQ16, ldC16;  // row strides in 16-byte units
-    int nQ, nC;
-    int selfJoin;  // queries and candidates are the same set: (i, i) is always a pair
-    int symmetric; // self-join only: compute tiles on and above the diagonal, emit (q,c) and (c,q)
-    int nSlabs;
-    float eps2;
-    const float* sumsQ;
-    const float* sumsC;
-    unsigned long long* counters;
-    int2* pairs;
-    unsigned long long cap;
-    Raster raster;
-};
-
-// Distance test of one wave's 128x64 block of accumulators.  acc[fi][fj] is a 16x16 MFMA block:
-// lane l holds column l%16 and rows 4*(l/16) .. +3, i.e. 4 elements per block.
-//
-// The accumulators start at -(s_q + s_c)/2 instead of 0, so what arrives here is
-//     a = q.c - (s_q + s_c)/2 = -dist^2 / 2
-// and the reference's test  s_q + s_c - 2 q.c <= eps^2  (source/warpMma.cuh:241-257) reads
-//     a >= -eps^2/2,
-// one threshold for every element, exact in FP32 (the scaling by 2 is exact), and symmetric in q and c
-// like the reference's.  Screening, about 1/2 VALU op per element: the maximum of the lane's 128 elements
-// (formed per row of blocks) against the threshold; a wave in which no lane has a hit is done.  Otherwise
-// the rows of blocks with a hit somewhere in the wave yield their per-element bits, branch-free.
-//
-// kEdge: the tile touches the diagonal of a self-join or the ragged end of a dataset; self pairs are
-// forced and padded rows/cols are masked (source/warpMma.cuh:257-259).
-// Returns per-lane hit bits, shifted in from the right in evaluation order: element e = (fi&1)*16 + fj*4 + r
-// of the pair of row blocks fi/2 ends up in bit 31 - e of mask[fi/2].
-template <bool kEdge>
-__device__ __forceinline__ void test_block(const floatx4 (&acc)[kFragRows][kFragCols], const int (&cand)[kFragCols],
-                                           int qBase, int quad, int nQ, int nC, int selfJoin, float thr,
-                                           unsigned (&mask)[kFragRows / 2]) {
-    if (kEdge) {
-#pragma unroll
-        for (int fp = 0; fp < kFragRows / 2; ++fp) {
-            unsigned m = 0;
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int fi = fp * 2 + h;
-#pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int q = qBase + fi * 16 + quad * 4 + r;
-                        const bool hit =
-                            (acc[fi][fj][r] >= thr || (selfJoin && q == cand[fj])) && q < nQ && cand[fj] < nC;
-                        m = (m << 1) | (hit ? 1u : 0u);
-                    }
-                }
-            }
-            mask[fp] = m;
-        }
-        return;
-    }
-    // maximum of every row of blocks (16 elements per lane), then of all of them
-    float rowBest[kFragRows];
-#pragma unroll
-    for (int fi = 0; fi < kFragRows; ++fi) {
-        float best = acc[fi][0][0];
-#pragma unroll
-        for (int fj = 0; fj < kFragCols; ++fj)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) best = __builtin_fmaxf(best, acc[fi][fj][r]);
-        rowBest[fi] = best;
-    }
-    float best = rowBest[0];
-#pragma unroll
-    for (int fi = 1; fi < kFragRows; ++fi) best = __builtin_fmaxf(best, rowBest[fi]);
-    if (__builtin_amdgcn_ballot_w64(best >= thr) == 0ull) {
-#pragma unroll
-        for (int fp = 0; fp < kFragRows / 2; ++fp) mask[fp] = 0u;
-        return;
-    }
-    // some lane has a hit: rows of blocks without one (wave-wide) are skipped, the others yield their
-    // bits: the sign of acc - thr (set = no hit) is shifted in; the maximum with -inf turns a NaN
-    // (points with infinite coordinates) into "no hit", as every comparison with NaN is false
-    unsigned long long rowHit[kFragRows];
-#pragma unroll
-    for (int fi = 0; fi < kFragRows; ++fi) rowHit[fi] = __builtin_amdgcn_ballot_w64(rowBest[fi] >= thr);
-#pragma unroll
-    for (int fp = 0; fp < kFragRows / 2; ++fp) {
-        unsigned m = 0;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int fi = fp * 2 + h;
-            if (rowHit[fi] != 0ull) {
-#pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        m = __builtin_amdgcn_alignbit(
-                            m, __builtin_bit_cast(unsigned, __builtin_fmaxf(acc[fi][fj][r], -__builtin_inff()) - thr), 31);
-            } else {
-                m = (m << 16) | 0xffffu;
-            }
-        }
-        mask[fp] = ~m;
-    }
-}
-
-// Lane number 0..63, re-derived from the execution mask where it is needed.  Volatile on purpose: the
-// optimiser then cannot hoist it (and what is derived from it) out of the tile loop, where it would
-// occupy registers, or spill, across the k loop.
-__device__ __forceinline__ int lane_now() {
-    int l;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-    return l;
-}
-
 template <bool kEpilogue>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __shared__ __align__(16) unsigned char lds[kLdsBytes];
@@ -568,9 +405,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
             unsigned mask[kFragRows / 2];
             if (edge)
-                test_block<true>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
+                test_block<kFragRows, kFragCols, true>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
             else
-                test_block<false>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
+                test_block<kFragRows, kFragCols, false>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
 
             // symmetric mode: a tile above the diagonal also stands for its mirror image
             const bool mirror = p.symmetric && tr != tc;
@@ -712,7 +549,7 @@ hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned l
     return hipGetLastError();
 }
 
-hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
+hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     static int numCUs = 0;
     static bool configured = false;
     if (!configured) {
@@ -725,6 +562,9 @@ hipError_t launch_join(const JoinLaunch& l, hipStream_t stream) {
         numCUs = prop.multiProcessorCount;
         configured = true;
     }
+    JoinLaunch l = launch;
+    // the kernels compare against -eps^2/2 and rely on that threshold being finite
+    if (!(l.eps2 < 3.0e38f)) l.eps2 = 3.0e38f;
     JoinParams p;
     p.ptsQ = static_cast<const u32x4*>(l.queries);
     p.ptsC = static_cast<const u32x4*>(l.candidates);
