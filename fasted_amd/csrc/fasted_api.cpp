@@ -55,28 +55,33 @@ bool quiet() {
     return q;
 }
 
-// Small device workspace that survives between calls: counters and a squared-norm buffer.
+// Small device workspace that survives between calls: counters, a squared-norm buffer and the buffer of
+// per-point accumulator start values (eps^2/4 - s/2) that the join kernel reads.
 struct Workspace {
     unsigned long long* counters = nullptr;
     float* sums = nullptr;
-    size_t sumsCap = 0;
+    float* halves = nullptr;
+    size_t cap = 0;
 
     void ensure(size_t n) {
         if (!counters) HIP_CHECK(hipMalloc(&counters, fasted::counter_words() * sizeof(unsigned long long)));
-        if (n > sumsCap) {
+        if (n > cap) {
             if (sums) HIP_CHECK(hipFree(sums));
-            sums = nullptr;
-            sumsCap = 0;
+            if (halves) HIP_CHECK(hipFree(halves));
+            sums = halves = nullptr;
+            cap = 0;
             HIP_CHECK(hipMalloc(&sums, n * sizeof(float)));
-            sumsCap = n;
+            HIP_CHECK(hipMalloc(&halves, n * sizeof(float)));
+            cap = n;
         }
     }
     void release() {
         if (counters) (void)hipFree(counters);
         if (sums) (void)hipFree(sums);
+        if (halves) (void)hipFree(halves);
         counters = nullptr;
-        sums = nullptr;
-        sumsCap = 0;
+        sums = halves = nullptr;
+        cap = 0;
     }
 } g_ws;
 
@@ -85,9 +90,9 @@ struct Workspace {
 // the counter block (pair counter + queue heads) and the squared norms.  They live in one file-scope device
 // array instead of hipMalloc'ed memory; each GPU the library runs on holds its own copy at its own address,
 // looked up once per device.  Host code never uses the array's name as an address: only `base`.
-constexpr size_t kNoAllocMaxPoints = (size_t)1 << 22;  // 4 Mi points: 16 MiB of squared norms
+constexpr size_t kNoAllocMaxPoints = (size_t)1 << 22;  // 4 Mi points: 2 x 16 MiB (squared norms, accumulator start values)
 constexpr size_t kNoAllocCounterBytes = 4096;          // counter block (1152 bytes used)
-constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + kNoAllocMaxPoints * sizeof(float);
+constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + 2 * kNoAllocMaxPoints * sizeof(float);  // norms, halves
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
 constexpr int kMaxDevices = 64;
@@ -117,6 +122,7 @@ DeviceScratch& device_scratch() {
 struct JoinScratch {
     unsigned long long* counters;
     float* sums;
+    float* halves;
     hipEvent_t* ev;  // three events
 };
 
@@ -178,23 +184,35 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     EventTimer t(fixed ? fixed->ev : nullptr);
     unsigned long long* counters = nullptr;
     float* wsSums = nullptr;
+    float* wsHalves = nullptr;
     if (fixed) {
         counters = fixed->counters;
         wsSums = fixed->sums;
+        wsHalves = fixed->halves;
     } else {
         g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
         counters = g_ws.counters;
         wsSums = g_ws.sums;
+        wsHalves = g_ws.halves;
     }
     float* sumsQ = q.sums ? q.sums : wsSums;
     float* sumsC = selfJoin ? sumsQ : (c.sums ? c.sums : wsSums + q.n);
+    float* halfQ = wsHalves;
+    float* halfC = selfJoin ? halfQ : wsHalves + q.n;
     if ((flags & FASTED_SKIP_SUMS) && (!q.sums || (!selfJoin && !c.sums)))
         throw std::invalid_argument("FASTED_SKIP_SUMS needs the squared-norm buffers");
+    const float eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
 
+    // squared norms and, from them, each point's accumulator start value eps^2/4 - s/2
     HIP_CHECK(hipEventRecord(t.ev[0], stream));
+    HIP_CHECK(fasted::launch_reset_counters(counters, false, stream));
     if (!(flags & FASTED_SKIP_SUMS)) {
-        HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, stream));
-        if (!selfJoin) HIP_CHECK(fasted::launch_sum_squared(c.ptr, c.ld, (int)c.n, dPad, sumsC, stream));
+        HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, halfQ, eps2, counters, stream));
+        if (!selfJoin)
+            HIP_CHECK(fasted::launch_sum_squared(c.ptr, c.ld, (int)c.n, dPad, sumsC, halfC, eps2, counters, stream));
+    } else {
+        HIP_CHECK(fasted::launch_halves(sumsQ, (int)q.n, eps2, halfQ, counters, stream));
+        if (!selfJoin) HIP_CHECK(fasted::launch_halves(sumsC, (int)c.n, eps2, halfC, counters, stream));
     }
     HIP_CHECK(hipEventRecord(t.ev[1], stream));
 
@@ -208,14 +226,12 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.selfJoin = selfJoin;
     jl.symmetric = selfJoin && (flags & FASTED_SYMMETRIC);
     jl.dPad = dPad;
-    jl.eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
-    jl.sumsQ = sumsQ;
-    jl.sumsC = sumsC;
+    jl.halfQ = halfQ;
+    jl.halfC = halfC;
     jl.counters = counters;
     jl.pairs = dPairs;
     jl.cap = cap;
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
-    HIP_CHECK(fasted::launch_reset_counters(counters, false, stream));
     HIP_CHECK(fasted::launch_join(jl, stream));
     HIP_CHECK(hipEventRecord(t.ev[2], stream));
     HIP_CHECK(hipStreamSynchronize(stream));
@@ -323,6 +339,7 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
     HIP_CHECK(hipStreamCreateWithFlags(&dev.copy, hipStreamNonBlocking));
     void* qBlock = dev.alloc(blockBytes);
     void* cBlock[2] = {dev.alloc(blockBytes), dev.alloc(blockBytes)};
+    // per-point accumulator start values of the query block and of the two candidate buffers
     float* qSums = static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)));
     float* cSums[2] = {static_cast<float*>(dev.alloc((size_t)rows * sizeof(float))),
                        static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)))};
@@ -344,8 +361,8 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
     for (long long i = 0; i < blocks; ++i) {
         const int nQ = (int)block_rows(i);
         upload(qBlock, i, dev.compute);
-        HIP_CHECK(fasted::launch_sum_squared(qBlock, dPad, nQ, dPad, qSums, dev.compute));
         HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, dev.compute));
+        HIP_CHECK(fasted::launch_sum_squared(qBlock, dPad, nQ, dPad, nullptr, qSums, eps2, g_ws.counters, dev.compute));
         unsigned long long before = 0;  // pairs of this query block found so far
         // candidate blocks other than block i itself pass through the two buffers in turn; `nextUp` is the
         // block to upload next, cBlock[slot] the buffer the next such join reads
@@ -366,7 +383,8 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
                 cand = cBlock[slot];
                 candSums = cSums[slot];
                 nC = (int)block_rows(j);
-                HIP_CHECK(fasted::launch_sum_squared(cand, dPad, nC, dPad, cSums[slot], dev.compute));
+                HIP_CHECK(fasted::launch_sum_squared(cand, dPad, nC, dPad, nullptr, cSums[slot], eps2, g_ws.counters,
+                                                     dev.compute));
             }
             fasted::JoinLaunch jl;
             jl.queries = qBlock;
@@ -377,9 +395,8 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
             jl.selfJoin = diagonal;
             jl.symmetric = false;
             jl.dPad = dPad;
-            jl.eps2 = eps2;
-            jl.sumsQ = qSums;
-            jl.sumsC = candSums;
+            jl.halfQ = qSums;
+            jl.halfC = candSums;
             jl.counters = g_ws.counters;
             jl.pairs = dPairs;
             jl.cap = devCap;
@@ -786,8 +803,8 @@ int fasted_self_join_device_noalloc(const void* d_points, long long n, int d, lo
         if (flags & FASTED_SKIP_SUMS)
             throw std::invalid_argument("fasted_self_join_device_noalloc computes the squared norms itself");
         DeviceScratch& ds = device_scratch();
-        const JoinScratch js{reinterpret_cast<unsigned long long*>(ds.base),
-                             reinterpret_cast<float*>(ds.base + kNoAllocCounterBytes), ds.ev};
+        float* const norms = reinterpret_cast<float*>(ds.base + kNoAllocCounterBytes);
+        const JoinScratch js{reinterpret_cast<unsigned long long*>(ds.base), norms, norms + kNoAllocMaxPoints, ds.ev};
         const PointSet all{d_points, n, ld, nullptr};
         join_on_device(all, all, true, d, epsilon, d_pairs, cap, flags, static_cast<hipStream_t>(stream), stats, &js);
     });
@@ -824,8 +841,8 @@ int fasted_sum_squared_device(const void* d_points, long long n, int d, long lon
     return guarded([&] {
         if (!d_points || !d_sums) throw std::invalid_argument("null pointer");
         validate_shape(n, d, ld);
-        HIP_CHECK(fasted::launch_sum_squared(d_points, ld, (int)n, round_up(d, fasted::kSlabK), d_sums,
-                                             static_cast<hipStream_t>(stream)));
+        HIP_CHECK(fasted::launch_sum_squared(d_points, ld, (int)n, round_up(d, fasted::kSlabK), d_sums, nullptr, 0.0f,
+                                             nullptr, static_cast<hipStream_t>(stream)));
         HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     });
 }

@@ -18,9 +18,8 @@ struct JoinLaunch {
     bool selfJoin;               // same set on both sides: (i, i) always counts as a pair
     bool symmetric;              // self-join: only tiles on/above the diagonal are computed, pairs mirrored
     int dPad;                    // K extent, multiple of kSlabK
-    float eps2;                  // (float)(eps*eps), source/findPairs.cuh:678
-    const float* sumsQ;          // squared norms of the queries
-    const float* sumsC;          // ... of the candidates
+    const float* halfQ;          // per query point: eps^2/4 - s/2 (s = squared norm), see launch_sum_squared
+    const float* halfC;          // ... per candidate point
     unsigned long long* counters;  // counter_words() words: [0] pairs found, then the queue heads
     void* pairs;                 // FastedPair[cap]
     unsigned long long cap;
@@ -36,8 +35,16 @@ unsigned long long tile_count(long long nQ, long long nC);  // 256x256 tiles the
 // Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).
 int lds_chunk_slot(int row, int chunk);
 
-hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream);
-// Clears the queue heads and, unless keepFound, the pair counter (word 0 of `counters`).
+// Squared norms of n points into `sums` (may be null) and, when `halves` is given, the per-point start value of
+// the join's accumulators  h = eps2/4 - s/2  (eps2 = (float)(eps*eps), source/findPairs.cuh:678): the join kernel
+// tests  h_q + h_c + q.c >= 0.  A non-finite norm raises the flag in `counters` (the join then tests element
+// by element), so the counters must have been reset before.
+hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, float* halves, float eps2,
+                              unsigned long long* counters, hipStream_t stream);
+// The same halves from norms that are already there.
+hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, unsigned long long* counters,
+                         hipStream_t stream);
+// Clears the queue heads and, unless keepFound, the pair counter and the non-finite flag (words 0, 1 of `counters`).
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream);
 // pairs[first, last): QueryPoint += qOffset, CandidatePoint += cOffset.
 hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,

@@ -42,10 +42,9 @@ constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 
 constexpr int kLdsSums = 2 * kStageBytes;           // two buffers of s_q[256] then s_c[256] (current / next tile)
 constexpr int kSumsBytes = 2 * kTile * 4;
 constexpr int kLdsNext = kLdsSums + 2 * kSumsBytes; // next tile of this workgroup: (row, col) as two u32
-constexpr int kLdsStageCount = kLdsNext + 16;       // pairs waiting in the LDS staging area (u32) + flush base (u64)
-constexpr int kLdsStage = kLdsStageCount + 16;      // staged pairs
-constexpr int kStagePairs = 3072;                   // 24 KiB of 8-byte records
-constexpr int kLdsBytes = kLdsStage + kStagePairs * 8;
+constexpr int kLdsStage = kLdsNext + 16;            // staged pairs: one private region per wave
+constexpr int kWaveStagePairs = 384;                // 3 KiB of 8-byte records per wave
+constexpr int kLdsBytes = kLdsStage + 8 * kWaveStagePairs * 8;
 static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
@@ -73,9 +72,12 @@ __host__ __device__ inline void raster_decode(const Raster& r, unsigned q, unsig
 }
 
 // ------------------------------------------------------------------------------------------
+// Optionally also writes, per point, h = quarterEps2 - s/2 (what the join kernel starts its accumulators
+// from) and raises the non-finite flag of the counter block when a squared norm is infinite or NaN.
 __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restrict__ pts, long long ld16, int n,
                                                           int chunksPerRow, int lanesPerRow,
-                                                          float* __restrict__ sums) {
+                                                          float* __restrict__ sums, float* __restrict__ halves,
+                                                          float quarterEps2, unsigned long long* __restrict__ counters) {
     const int lane = threadIdx.x & 63;
     const long long wave = ((long long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int rowsPerWave = 64 / lanesPerRow;
@@ -111,13 +113,30 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
         acc = (part[0] + part[1]) + (part[2] + part[3]);
     }
     for (int off = lanesPerRow >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (sub == 0 && row < n) sums[row] = acc;
+    if (sub == 0 && row < n) {
+        if (sums) sums[row] = acc;
+        if (halves) {
+            halves[row] = __builtin_fmaf(acc, -0.5f, quarterEps2);
+            if (!(__builtin_fabsf(acc) < __builtin_inff())) counters[kCounterNonFinite] = 1ull;
+        }
+    }
 }
 
-// Clears the queue heads and, unless `keepFound`, the pair counter (word 0): a launch that keeps it
-// appends its pairs behind those of the launch before.
+// The same per-point halves from squared norms that are already there.
+__global__ void __launch_bounds__(256) halves_kernel(const float* __restrict__ sums, int n, float quarterEps2,
+                                                     float* __restrict__ halves, unsigned long long* __restrict__ counters) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float s = sums[i];
+    halves[i] = __builtin_fmaf(s, -0.5f, quarterEps2);
+    if (!(__builtin_fabsf(s) < __builtin_inff())) counters[kCounterNonFinite] = 1ull;
+}
+
+// Clears the queue heads and, unless `keepFound`, the pair counter (word 0) and the non-finite flag (word 1):
+// a launch that keeps them appends its pairs behind those of the launch before.
 __global__ void reset_counters_kernel(unsigned long long* c, int keepFound) {
-    if (threadIdx.x < kCounterWords && !(keepFound && threadIdx.x == kCounterFound)) c[threadIdx.x] = 0ull;
+    if (threadIdx.x < kCounterWords && !(keepFound && (threadIdx.x == kCounterFound || threadIdx.x == kCounterNonFinite)))
+        c[threadIdx.x] = 0ull;
 }
 
 // Adds the first row of the query block and of the candidate block to the pairs [first, last) that a
@@ -134,6 +153,14 @@ __global__ void __launch_bounds__(256) offset_pairs_kernel(int2* pairs, unsigned
 }
 
 // ------------------------------------------------------------------------------------------
+// The barrier of the tile loop: every global->LDS transfer this wave has issued has landed (they are vector
+// memory operations: vmcnt), every LDS operation of the wave is complete, then the workgroup meets.  Written
+// out because the wait is part of the algorithm: __syncthreads() only promises the LDS counter at workgroup
+// scope, and the compiler does not track what a buffer-form transfer writes to LDS.
+__device__ __forceinline__ void transfers_landed_barrier() {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <bool kEpilogue>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __shared__ __align__(16) unsigned char lds[kLdsBytes];
@@ -157,9 +184,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // LDS byte address of lds[0], for the LDS instructions written out by hand below
     const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
     unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // next tile: [0] row, [1] col
-    unsigned* const sStageCount = reinterpret_cast<unsigned*>(lds + kLdsStageCount);
-    unsigned long long* const sFlushBase = reinterpret_cast<unsigned long long*>(lds + kLdsStageCount + 8);
-    int2* const sStage = reinterpret_cast<int2*>(lds + kLdsStage);
+    const int2* const sStage = reinterpret_cast<const int2*>(lds + kLdsStage) + wave * kWaveStagePairs;  // this wave's region
+
+    // set by the kernel that formed the per-point halves: some point has a non-finite squared norm
+    const bool nonFinite = p.counters[kCounterNonFinite] != 0ull;
 
     // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
     const unsigned home = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (kQueues - 1);
@@ -194,57 +222,76 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         }
     };
 
-    // Pairs are staged in LDS and appended to the global list by the whole workgroup: one
-    // reservation on the global counter per flush instead of one per wave and tile, which is what
-    // bounds output-heavy joins (same-address atomics serialise at about 12 ns each).
-    auto flush_stage = [&](unsigned staged) {
-        const unsigned cnt = staged < (unsigned)kStagePairs ? staged : (unsigned)kStagePairs;
-        const unsigned tid = (unsigned)(wave * 64 + lane_now());
-        if (tid == 0) *sFlushBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)cnt);
-        __syncthreads();
-        const unsigned long long gb = *sFlushBase;
-        for (unsigned i = tid; i < cnt; i += kThreads)
-            if (gb + i < p.cap) p.pairs[gb + i] = sStage[i];  // past the capacity: counted, not stored
-        __syncthreads();
-        if (tid == 0) *sStageCount = 0u;
-        __syncthreads();
+    // Pairs are staged in LDS, in a region private to each wave whose fill count lives in a scalar
+    // register: appending needs no atomic and no barrier.  A region goes to the global list with one
+    // reservation on the global counter (same-address atomics serialise at about 12 ns each: one per pair,
+    // or per wave and tile, is what would bound output-heavy joins) and coalesced 8-byte stores.
+    int staged = 0;
+    auto flush_wave = [&]() {
+        const int ln = lane_now();
+        unsigned long long base = 0;
+        if (ln == 0) base = atomicAdd(&p.counters[kCounterFound], (unsigned long long)staged);
+        base = ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(base >> 32)) << 32) |
+               __builtin_amdgcn_readfirstlane((unsigned)base);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staged records are in LDS
+        for (int i = ln; i < staged; i += 64)
+            if (base + i < p.cap) p.pairs[base + i] = sStage[i];  // past the capacity: counted, not stored
+        staged = 0;
     };
 
     // Byte offsets, from the tile's first row, of the 16-byte chunks this lane copies: 4 query rows and
-    // 4 candidate rows per slab.  Rows past the end of the dataset re-read the last real row; their
-    // results are masked.  The swizzle is applied here, on the global side.
-    auto tile_offsets = [&](int rowBase, int colBase, unsigned (&oA)[4], unsigned (&oB)[4]) {
+    // 4 candidate rows per slab.  The swizzle is applied here, on the global side.  Rows past the end of
+    // the dataset re-read the last real row (their results are masked), so only the ragged last tiles have
+    // offsets of their own: the offsets are formed again only when a ragged tile comes or goes.
+    bool clampedA = false, clampedB = false;  // the current offsets belong to a ragged tile
+    auto side_offsets = [&](int base, int n, long long ld16, unsigned (&o)[4]) {
         const int ln = lane_now();
         const int row0 = wave * 32 + (ln >> 3);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = row0 + 8 * i;
             const int chunk = (ln & 7) ^ swz(r);
-            oA[i] = (unsigned)(min(r, p.nQ - 1 - rowBase) * (int)p.ldQ16 + chunk) * 16u;
-            oB[i] = (unsigned)(min(r, p.nC - 1 - colBase) * (int)p.ldC16 + chunk) * 16u;
+            o[i] = (unsigned)(min(r, n - 1 - base) * (int)ld16 + chunk) * 16u;
+        }
+    };
+    auto tile_offsets = [&](int rowBase, int colBase, unsigned (&oA)[4], unsigned (&oB)[4], bool first) {
+        const bool raggedA = rowBase + kTile > p.nQ, raggedB = colBase + kTile > p.nC;
+        if (first || raggedA || clampedA) {
+            side_offsets(rowBase, p.nQ, p.ldQ16, oA);
+            clampedA = raggedA;
+        }
+        if (first || raggedB || clampedB) {
+            side_offsets(colBase, p.nC, p.ldC16, oB);
+            clampedB = raggedB;
         }
     };
 
     // One 1-KiB global->LDS transfer of this wave (global_load_lds_dwordx4: no registers in between);
     // j = 0..7 alternates query / candidate rows.  Lane l lands in row l/8, chunk slot l%8 of the
     // 8 rows the instruction fills; wave w owns rows [32w, 32w+32) of both operands.
-    auto issue_load = [&](const char* gA, const char* gB, const unsigned (&oA)[4], const unsigned (&oB)[4],
-                          unsigned slabByte, int stage, int j) {
+    auto issue_load = [&](__amdgpu_buffer_rsrc_t rA, __amdgpu_buffer_rsrc_t rB, const unsigned (&oA)[4],
+                          const unsigned (&oB)[4], int slabByte, int stage, int j) {
         const int i = j >> 1;
         unsigned char* const dst = lds + stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes;
-        // uniform 64-bit base + 32-bit lane offset (formed here so it stays a 32-bit add)
-        const char* const src = (j & 1) ? gB + (oB[i] + slabByte) : gA + (oA[i] + slabByte);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        // buffer form of the transfer: the tile's first row is the buffer base (scalar registers), the lane's
+        // offset a 32-bit vector register that never changes, the slab's offset a scalar register: no vector
+        // arithmetic per transfer
+        __builtin_amdgcn_raw_ptr_buffer_load_lds((j & 1) ? rB : rA, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 (int)((j & 1) ? oB[i] : oA[i]), slabByte, 0, 0);
+    };
+    // Buffer descriptor over the rows of one operand of a tile.  The range check is left wide open: rows and
+    // columns are clamped into the dataset when the offsets are formed.
+    auto tile_buffer = [&](const u32x4* base) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(base), 0, -1, 0x00020000);
     };
 
-    // Squared norms of a tile's 256 queries (waves 0-3) and 256 candidates (waves 4-7), 64 floats per
-    // wave, straight into the sums buffer `which`.
+    // Per-point halves (eps^2/4 - s/2) of a tile's 256 queries (waves 0-3) and 256 candidates (waves 4-7),
+    // 64 floats per wave, straight into the buffer `which`.
     auto issue_sums = [&](int rowBase, int colBase, int which) {
         const int ln = lane_now();
         const int part = wave & 3;
-        const float* src = wave < 4 ? p.sumsQ + min(rowBase + part * 64 + ln, p.nQ - 1)
-                                    : p.sumsC + min(colBase + part * 64 + ln, p.nC - 1);
+        const float* src = wave < 4 ? p.halfQ + min(rowBase + part * 64 + ln, p.nQ - 1)
+                                    : p.halfC + min(colBase + part * 64 + ln, p.nC - 1);
         unsigned char* const dst = lds + kLdsSums + which * kSumsBytes + wave * 256;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
@@ -252,7 +299,6 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     // ---- first tile
     if (wave == 0 && lane_now() == 0) {
-        *sStageCount = 0u;
         unsigned r, c;
         find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r, &c);
         sNext[0] = r;
@@ -265,11 +311,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __syncthreads();  // everybody has read sNext before thread 0 writes the second tile there
 
     unsigned offA[4], offB[4];
-    tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB);
-    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)tr * kTile * p.ldQ16);
-    const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)tc * kTile * p.ldC16);
+    tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB, true);
+    __amdgpu_buffer_rsrc_t gA = tile_buffer(p.ptsQ + (long long)tr * kTile * p.ldQ16);
+    __amdgpu_buffer_rsrc_t gB = tile_buffer(p.ptsC + (long long)tc * kTile * p.ldC16);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0u, 0, j);
+    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0, 0, j);
     issue_sums((int)tr * kTile, (int)tc * kTile, 0);
     unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
     if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
@@ -279,11 +325,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     for (;;) {
         // slab 0 of this tile (issued during the previous tile's last slab) has landed
-        __syncthreads();
-        if (kEpilogue) {
-            const unsigned staged = __builtin_amdgcn_readfirstlane(*sStageCount);
-            if (staged >= (unsigned)kStagePairs / 2) flush_stage(staged);
-        }
+        transfers_landed_barrier();
         if (wave == 0 && lane_now() == 0) {
             // the reservation made a whole tile ago has long arrived: no wait here
             unsigned r, c;
@@ -293,8 +335,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         }
 
-        // the accumulators start at -(s_q + s_c)/2 (see test_block): the tile's squared norms landed
-        // together with slab 0
+        // the accumulators start at h_q + h_c, h = eps^2/4 - s/2 per point (see the epilogue): the tile's
+        // 512 values landed together with slab 0
         floatx4 acc[kFragRows][kFragCols];
         {
             const int ln = lane_now();
@@ -304,12 +346,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + kTile + wc * kWaveCols + (ln & 15);
             float hc[kFragCols];
 #pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj) hc[fj] = -0.5f * sCw[fj * 16];
+            for (int fj = 0; fj < kFragCols; ++fj) hc[fj] = sCw[fj * 16];
 #pragma unroll
             for (int fi = 0; fi < kFragRows; ++fi) {
-                const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16) * -0.5f;
+                const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16);
 #pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) acc[fi][fj] = hq + hc[fj];
+                for (int fj = 0; fj < kFragCols; ++fj) acc[fi][fj] = hq + hc[fj];  // commutative: the same for (q, c) and (c, q)
             }
         }
 
@@ -322,10 +364,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // 4 MFMAs during the first k-step: spaced so that the texture-address queue never makes a
         // wave wait with the matrix pipe idle, early so that an L2 miss has the whole second
         // k-step to land before the slab's barrier.
-        auto slab_step = [&](int stg, bool prefetch, const char* pA, const char* pB, const unsigned (&oA)[4],
-                             const unsigned (&oB)[4], unsigned nextByte) {
+        auto slab_step = [&](int stg, bool prefetch, __amdgpu_buffer_rsrc_t pA, __amdgpu_buffer_rsrc_t pB,
+                             const unsigned (&oA)[4], const unsigned (&oB)[4], int nextByte) {
             const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[4], aHi[4], b[2][kFragCols];
+
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
                 b[0][fj] = *reinterpret_cast<const half8*>(buf + bOff[0] + fj * 16 * kRowBytes);
@@ -372,11 +415,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         };
 
         for (int s = 0; s + 1 < p.nSlabs; ++s) {
-            slab_step(stage, true, gA, gB, offA, offB, (unsigned)(s + 1) * kRowBytes);
+            slab_step(stage, true, gA, gB, offA, offB, (s + 1) * kRowBytes);
             stage ^= 1;
-            __syncthreads();
+            transfers_landed_barrier();
         }
-        if (p.nSlabs == 1) __syncthreads();  // with a single slab no barrier has published sNext yet
+        if (p.nSlabs == 1) transfers_landed_barrier();  // with a single slab no barrier has published sNext yet
 
         // The tile after this one: its first slab and its squared norms travel during this tile's last
         // slab and epilogue.  The current tile's offsets are not needed any more, so the next tile's
@@ -385,94 +428,132 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const unsigned ntc = __builtin_amdgcn_readfirstlane(sNext[1]);
         const bool more = ntr != kNoTile;
         if (more) {
-            tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB);
-            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
-            gB = reinterpret_cast<const char*>(p.ptsC + (long long)ntc * kTile * p.ldC16);
+            tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB, false);
+            gA = tile_buffer(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
+            gB = tile_buffer(p.ptsC + (long long)ntc * kTile * p.ldC16);
             issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
         }
-        slab_step(stage, more, gA, gB, offA, offB, 0u);
+        slab_step(stage, more, gA, gB, offA, offB, 0);
         stage ^= 1;
 
         if (kEpilogue) {
+            // Fused test (source/warpMma.cuh:220-273).  The accumulators started at h_q + h_c with
+            // h = eps^2/4 - s/2 per point, so an element now holds a = q.c - (s_q + s_c)/2 + eps^2/2 =
+            // (eps^2 - dist^2)/2 and the reference's test  s_q + s_c - 2 q.c <= eps^2  reads  a >= 0: the sign
+            // bit of the accumulator, symmetric in q and c like the reference's test.
             const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
             const int ln = lane_now();
-            const int l16 = ln & 15, quad = ln >> 4;
-            const int qBase = rowBase + wr * kWaveRows;
-            int cand[kFragCols];
-#pragma unroll
-            for (int fj = 0; fj < kFragCols; ++fj) cand[fj] = colBase + wc * kWaveCols + fj * 16 + l16;
-            const float thr = -0.5f * p.eps2;
-            const bool edge = (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
-            unsigned mask[kFragRows / 2];
-            if (edge)
-                test_block<kFragRows, kFragCols, true>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
-            else
-                test_block<kFragRows, kFragCols, false>(acc, cand, qBase, quad, p.nQ, p.nC, p.selfJoin, thr, mask);
+            const int qLane = rowBase + wr * kWaveRows + (ln >> 4) * 4;  // row of element r = 0 of block row 0
+            const int cLane = colBase + wc * kWaveCols + (ln & 15);      // column in block column 0
+            // Every element is tested one by one when the tile touches the diagonal of a self-join or the ragged
+            // end of a dataset (self pairs are forced, padded rows/columns masked: source/warpMma.cuh:257-259)
+            // or when the dataset holds points with non-finite norms (a NaN must compare as "no hit").
+            const bool edge = nonFinite || (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
+            const bool mirror = p.symmetric && tr != tc;  // a tile above the diagonal also stands for its mirror image
 
-            // symmetric mode: a tile above the diagonal also stands for its mirror image
-            const bool mirror = p.symmetric && tr != tc;
-            int mine = 0;
+            // Per-lane hit bits of the 4 pairs of block rows: element e = (fi & 1) * 16 + fj * 4 + r of the pair
+            // fi / 2 is bit 31 - e.
+            unsigned hits[kFragRows / 2];
+            bool any;
+            if (!edge) {
+                // Screening, about 1/2 vector instruction per element: the maximum of the lane's 128 elements,
+                // formed per row of blocks; a wave in which no lane has a hit is done.
+                float rowBest[kFragRows];
 #pragma unroll
-            for (int fp = 0; fp < kFragRows / 2; ++fp) mine += __builtin_popcount(mask[fp]);
-            if (mirror) mine *= 2;
-            if (__builtin_amdgcn_ballot_w64(mine != 0) != 0ull) {
-                // wave-level compaction: inclusive prefix sum of per-lane counts, one reservation
-                // (data-parallel-primitive moves inside the vector ALU: shifts within rows of 16 lanes, then the
-                // last lane of row 0/2 added to row 1/3, then lane 31 to the upper half)
-                int incl = mine;
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x111, 0xf, 0xf, false);  // row_shr:1
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x112, 0xf, 0xf, false);  // row_shr:2
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x114, 0xf, 0xf, false);  // row_shr:4
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x118, 0xf, 0xf, false);  // row_shr:8
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
-                incl += __builtin_amdgcn_update_dpp(0, incl, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
-                const unsigned total = (unsigned)__builtin_amdgcn_readlane(incl, 63);
-                // reserve room in the staging area (LDS atomic); what does not fit goes straight
-                // to the global list with a reservation of this wave's own
-                // (LDS atomic and LDS stores below are written as instructions: for ordinary LDS writes the
-                // compiler first waits until this wave's global->LDS transfers of the next tile have landed)
-                unsigned pos = 0;
-                if (ln == 0)
-                    asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
-                                 : "=v"(pos)
-                                 : "v"(ldsBase + (unsigned)kLdsStageCount), "v"(total)
-                                 : "memory");
-                pos = __builtin_amdgcn_readfirstlane(pos);
-                const unsigned room = pos < (unsigned)kStagePairs ? (unsigned)kStagePairs - pos : 0u;
-                const unsigned fit = total < room ? total : room;
-                unsigned long long gbase = 0;
-                if (fit < total) {
-                    if (ln == 0) gbase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)(total - fit));
-                    gbase = ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(gbase >> 32)) << 32) |
-                            __builtin_amdgcn_readfirstlane((unsigned)gbase);
+                for (int fi = 0; fi < kFragRows; ++fi) {
+                    float best = acc[fi][0][0];
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) best = __builtin_fmaxf(best, acc[fi][fj][r]);
+                    rowBest[fi] = best;
                 }
-                unsigned idx = (unsigned)(incl - mine);
+                float best = rowBest[0];
 #pragma unroll
-                for (int fp = 0; fp < kFragRows / 2; ++fp) {
-                    unsigned m = mask[fp];
-                    while (m) {
-                        const int low = __builtin_ctz(m);
-                        m &= m - 1;
-                        const int bit = 31 - low;  // element number inside the pair of row blocks
-                        const int fi = fp * 2 + (bit >> 4), fj = (bit >> 2) & 3, r = bit & 3;
-                        const int q = qBase + fi * 16 + quad * 4 + r;
-                        const int c = colBase + wc * kWaveCols + fj * 16 + l16;
-                        auto put = [&](unsigned at, int first, int second) {
-                            if (at < fit) {
-                                const unsigned long long rec =
-                                    (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
-                                asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage + (pos + at) * 8u), "v"(rec)
-                                             : "memory");
+                for (int fi = 1; fi < kFragRows; ++fi) best = __builtin_fmaxf(best, rowBest[fi]);
+                any = __builtin_amdgcn_ballot_w64(best >= 0.0f) != 0ull;
+                if (any) {
+                    // the rows of blocks with a hit somewhere in the wave yield their bits, one instruction per
+                    // element: the sign of the accumulator (set = no hit) is shifted in
+#pragma unroll
+                    for (int fp = 0; fp < kFragRows / 2; ++fp) {
+                        unsigned m = ~0u;
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int fi = fp * 2 + h;
+                            if (__builtin_amdgcn_ballot_w64(rowBest[fi] >= 0.0f) != 0ull) {
+#pragma unroll
+                                for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+                                    for (int r = 0; r < 4; ++r) {
+                                        const float a = acc[fi][fj][r];  // (a bit cast of the vector element itself reads element 0)
+                                        m = __builtin_amdgcn_alignbit(m, __float_as_uint(a), 31);
+                                    }
                             } else {
-                                const unsigned long long slot = gbase + (at - fit);
-                                if (slot < p.cap) p.pairs[slot] = make_int2(first, second);
+                                m = (m << 16) | 0xffffu;
                             }
-                        };
-                        put(idx++, q, c);
-                        if (mirror) put(idx++, c, q);
+                        }
+                        hits[fp] = ~m;
                     }
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staged records are in LDS
+            } else {
+                any = true;
+#pragma unroll
+                for (int fp = 0; fp < kFragRows / 2; ++fp) {
+                    unsigned m = 0u;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int fi = fp * 2 + h;
+#pragma unroll
+                        for (int fj = 0; fj < kFragCols; ++fj) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                const int q = qLane + fi * 16 + r, c = cLane + fj * 16;
+                                const bool hit =
+                                    ((acc[fi][fj][r] >= 0.0f) | ((p.selfJoin != 0) & (q == c))) & (q < p.nQ) & (c < p.nC);
+                                m = (m << 1) | (hit ? 1u : 0u);
+                            }
+                        }
+                    }
+                    hits[fp] = m;
+                }
+            }
+            if (any) {
+                // Extraction, one word of hit bits after the other.  Each round takes the first remaining hit
+                // of every lane that has one: the lanes form a mask in scalar registers, a lane's record goes
+                // behind those of the lanes before it, the wave's fill count moves on by the number of lanes.
+#pragma unroll 1
+                for (int fp = 0; fp < kFragRows / 2; ++fp) {
+                    unsigned w = fp == 0 ? hits[0] : fp == 1 ? hits[1] : fp == 2 ? hits[2] : hits[3];
+                    for (;;) {
+                        const unsigned long long lanes = __builtin_amdgcn_ballot_w64(w != 0u);
+                        if (lanes == 0ull) break;
+                        const int count = __builtin_popcountll(lanes) << (mirror ? 1 : 0);
+                        if (staged + count > kWaveStagePairs) flush_wave();
+                        if (w != 0u) {
+                            const int e = __builtin_clz(w);  // element number inside the pair of block rows
+                            w &= ~(0x80000000u >> e);
+                            const int q = qLane + fp * 32 + (e >> 4) * 16 + (e & 3);
+                            const int c = cLane + ((e >> 2) & 3) * 16;
+                            const unsigned before = __builtin_amdgcn_mbcnt_hi(
+                                (unsigned)(lanes >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)lanes, 0u));
+                            const unsigned at = (unsigned)staged + (mirror ? 2u * before : before);
+                            // written as an instruction: for an ordinary LDS store the compiler first waits until
+                            // this wave's global->LDS transfers of the next tile have landed
+                            auto put = [&](unsigned idx, int first, int second) {
+                                const unsigned long long rec =
+                                    (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
+                                asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage +
+                                                                         ((unsigned)wave * kWaveStagePairs + idx) * 8u),
+                                             "v"(rec)
+                                             : "memory");
+                            };
+                            put(at, q, c);
+                            if (mirror) put(at + 1, c, q);
+                        }
+                        staged += count;
+                    }
+                }
             }
         } else {
             // keep the accumulators observable without spending instructions on them
@@ -487,11 +568,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         tc = ntc;
         sumsBuf ^= 1;
     }
-    if (kEpilogue) {
-        __syncthreads();
-        const unsigned staged = __builtin_amdgcn_readfirstlane(*sStageCount);
-        if (staged > 0) flush_stage(staged);
-    }
+    if (kEpilogue && staged > 0) flush_wave();
 }
 
 }  // namespace
@@ -523,7 +600,11 @@ unsigned long long tile_count(long long nQ, long long nC) {
 
 int lds_chunk_slot(int row, int chunk) { return (chunk ^ swz(row)) & 7; }
 
-hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, hipStream_t stream) {
+// (float)(eps*eps) / 4, kept finite: the kernels rely on finite accumulator start values
+float quarter_eps2(float eps2) { return (eps2 < 3.0e38f ? eps2 : 3.0e38f) * 0.25f; }
+
+hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, float* halves, float eps2,
+                              unsigned long long* counters, hipStream_t stream) {
     const int chunksPerRow = dPad / 8;
     int lanesPerRow = 64;
     while (lanesPerRow > chunksPerRow) lanesPerRow >>= 1;
@@ -531,7 +612,14 @@ hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad,
     const long long waves = ((long long)n + rowsPerWave - 1) / rowsPerWave;
     const long long blocks = (waves + 3) / 4;
     sum_squared_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(static_cast<const u32x4*>(points), ld / 8, n,
-                                                                        chunksPerRow, lanesPerRow, sums);
+                                                                        chunksPerRow, lanesPerRow, sums, halves,
+                                                                        quarter_eps2(eps2), counters);
+    return hipGetLastError();
+}
+
+hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, unsigned long long* counters,
+                         hipStream_t stream) {
+    halves_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(sums, n, quarter_eps2(eps2), halves, counters);
     return hipGetLastError();
 }
 
@@ -562,9 +650,7 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
         numCUs = prop.multiProcessorCount;
         configured = true;
     }
-    JoinLaunch l = launch;
-    // the kernels compare against -eps^2/2 and rely on that threshold being finite
-    if (!(l.eps2 < 3.0e38f)) l.eps2 = 3.0e38f;
+    const JoinLaunch& l = launch;
     JoinParams p;
     p.ptsQ = static_cast<const u32x4*>(l.queries);
     p.ptsC = static_cast<const u32x4*>(l.candidates);
@@ -575,9 +661,8 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     p.selfJoin = l.selfJoin ? 1 : 0;
     p.symmetric = (l.selfJoin && l.symmetric) ? 1 : 0;
     p.nSlabs = l.dPad / kSlabK;
-    p.eps2 = l.eps2;
-    p.sumsQ = l.sumsQ;
-    p.sumsC = l.sumsC;
+    p.halfQ = l.halfQ;
+    p.halfC = l.halfC;
     p.counters = l.counters;
     p.pairs = static_cast<int2*>(l.pairs);
     p.cap = l.cap;
