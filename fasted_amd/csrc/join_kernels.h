@@ -52,8 +52,21 @@ hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned l
 hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
 
 
-// Row-major sort of `count` stored pairs (pair_sort.hip).
-hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream);
+// Device buffers of the row-major sort (a second key buffer and the radix sort's own storage).  They only
+// grow; a caller that keeps a SortBuffers across calls sorts without allocating.
+struct SortBuffers {
+    void* alt = nullptr;
+    size_t altBytes = 0;
+    void* temp = nullptr;
+    size_t tempBytes = 0;
+    void release();
+};
+// Row-major sort of `count` stored pairs (pair_sort.hip); synchronises the stream.  With ws == nullptr the
+// buffers are allocated and freed inside the call.  On failure (no memory for the buffers) the pairs are left
+// as they were, unsorted.
+hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws = nullptr);
+// Device bytes a sort of `count` pairs needs beside the pairs themselves.
+size_t sort_scratch_bytes(unsigned long long count);
 
 // out[i] = Euclidean distance of pair i (FP32 sum of squared differences over dPad dimensions); NaN for a
 // pair that names a point outside [0, nQ) x [0, nC).

@@ -46,6 +46,9 @@ constexpr int kLdsStage = kLdsNext + 16;            // staged pairs: one private
 constexpr int kWaveStagePairs = 384;                // 3 KiB of 8-byte records per wave
 constexpr int kLdsBytes = kLdsStage + 8 * kWaveStagePairs * 8;
 static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
+// false: the four transfers of half a k-step are issued in a cluster at its start (measured 1-3 % faster on
+// the 1M x 4096 workload than one transfer pinned in front of every 4 MFMAs)
+constexpr bool kSpread = false;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
@@ -154,11 +157,15 @@ __global__ void __launch_bounds__(256) offset_pairs_kernel(int2* pairs, unsigned
 
 // ------------------------------------------------------------------------------------------
 // The barrier of the tile loop: every global->LDS transfer this wave has issued has landed (they are vector
-// memory operations: vmcnt), every LDS operation of the wave is complete, then the workgroup meets.  Written
-// out because the wait is part of the algorithm: __syncthreads() only promises the LDS counter at workgroup
-// scope, and the compiler does not track what a buffer-form transfer writes to LDS.
+// memory operations: vmcnt), every LDS operation of the wave is complete, then the workgroup meets.  The wait
+// is written out because it is part of the algorithm: __syncthreads() alone only promises the LDS counter at
+// workgroup scope, and the transfers are hand-written instructions the compiler knows nothing about.  It is the
+// s_waitcnt builtin and not assembly text, so that the compiler's own bookkeeping of outstanding operations
+// sees it (behind an opaque wait it assumes the worst and waits for every LDS read of a slab before the first
+// MFMA).
 __device__ __forceinline__ void transfers_landed_barrier() {
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0), export counter left alone
+    __syncthreads();
 }
 
 template <bool kEpilogue>
@@ -269,20 +276,19 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // One 1-KiB global->LDS transfer of this wave (global_load_lds_dwordx4: no registers in between);
     // j = 0..7 alternates query / candidate rows.  Lane l lands in row l/8, chunk slot l%8 of the
     // 8 rows the instruction fills; wave w owns rows [32w, 32w+32) of both operands.
-    auto issue_load = [&](__amdgpu_buffer_rsrc_t rA, __amdgpu_buffer_rsrc_t rB, const unsigned (&oA)[4],
-                          const unsigned (&oB)[4], int slabByte, int stage, int j) {
+    auto issue_load = [&](const char* slabA, const char* slabB, const unsigned (&oA)[4], const unsigned (&oB)[4],
+                          int stage, int j) {
         const int i = j >> 1;
-        unsigned char* const dst = lds + stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes;
-        // buffer form of the transfer: the tile's first row is the buffer base (scalar registers), the lane's
-        // offset a 32-bit vector register that never changes, the slab's offset a scalar register: no vector
-        // arithmetic per transfer
-        __builtin_amdgcn_raw_ptr_buffer_load_lds((j & 1) ? rB : rA, (__attribute__((address_space(3))) void*)dst, 16,
-                                                 (int)((j & 1) ? oB[i] : oA[i]), slabByte, 0, 0);
-    };
-    // Buffer descriptor over the rows of one operand of a tile.  The range check is left wide open: rows and
-    // columns are clamped into the dataset when the offsets are formed.
-    auto tile_buffer = [&](const u32x4* base) {
-        return __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(base), 0, -1, 0x00020000);
+        const unsigned dst = ldsBase + (unsigned)(stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes);
+        // Written as instructions: the slab's address in scalar registers, the lane's offset a 32-bit vector
+        // register that never changes -- no vector arithmetic per transfer (left to the compiler, the
+        // addresses become loop-carried 64-bit vector pointers).  M0 holds the LDS destination.
+        if (j & 1)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(oB[i]), "s"(slabB)
+                         : "memory", "m0");
+        else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(oA[i]), "s"(slabA)
+                         : "memory", "m0");
     };
 
     // Per-point halves (eps^2/4 - s/2) of a tile's 256 queries (waves 0-3) and 256 candidates (waves 4-7),
@@ -312,10 +318,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     unsigned offA[4], offB[4];
     tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB, true);
-    __amdgpu_buffer_rsrc_t gA = tile_buffer(p.ptsQ + (long long)tr * kTile * p.ldQ16);
-    __amdgpu_buffer_rsrc_t gB = tile_buffer(p.ptsC + (long long)tc * kTile * p.ldC16);
+    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)tr * kTile * p.ldQ16);
+    const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)tc * kTile * p.ldC16);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0, 0, j);
+    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0, j);
     issue_sums((int)tr * kTile, (int)tc * kTile, 0);
     unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
     if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
@@ -360,12 +366,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // in snake order: consecutive MFMAs always share an operand, which the power-limited clock
         // rewards with about 1.5 %).  The instruction order is pinned with
         // scheduling barriers: the LDS reads for the next half are issued ahead of the MFMAs of
-        // the current half, and the 8 global->LDS transfers of the following slab are issued one per
-        // 4 MFMAs during the first k-step: spaced so that the texture-address queue never makes a
-        // wave wait with the matrix pipe idle, early so that an L2 miss has the whole second
-        // k-step to land before the slab's barrier.
-        auto slab_step = [&](int stg, bool prefetch, __amdgpu_buffer_rsrc_t pA, __amdgpu_buffer_rsrc_t pB,
-                             const unsigned (&oA)[4], const unsigned (&oB)[4], int nextByte) {
+        // the current half, and the 8 global->LDS transfers of the following slab are issued during
+        // the first k-step, four at the start of each of its halves: early, so that an L2 miss has the
+        // whole second k-step to land before the slab's barrier.
+        auto slab_step = [&](int stg, bool prefetch, const char* pA, const char* pB, const unsigned (&oA)[4],
+                             const unsigned (&oB)[4]) {
             const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[4], aHi[4], b[2][kFragCols];
 
@@ -383,12 +388,13 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi) {
-                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, fi);
+                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, stg ^ 1, fi);
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
                     }
+                    if (ks == 0 && kSpread) __builtin_amdgcn_sched_barrier(0);  // keeps each transfer in front of its 4 MFMAs
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -402,20 +408,21 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi) {
-                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, nextByte, stg ^ 1, 4 + fi);
+                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, stg ^ 1, 4 + fi);
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;
                         acc[fi + 4][fj] =
                             __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
                     }
+                    if (ks == 0 && kSpread) __builtin_amdgcn_sched_barrier(0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
 
         for (int s = 0; s + 1 < p.nSlabs; ++s) {
-            slab_step(stage, true, gA, gB, offA, offB, (s + 1) * kRowBytes);
+            slab_step(stage, true, gA + (s + 1) * kRowBytes, gB + (s + 1) * kRowBytes, offA, offB);
             stage ^= 1;
             transfers_landed_barrier();
         }
@@ -429,11 +436,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const bool more = ntr != kNoTile;
         if (more) {
             tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB, false);
-            gA = tile_buffer(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
-            gB = tile_buffer(p.ptsC + (long long)ntc * kTile * p.ldC16);
+            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
+            gB = reinterpret_cast<const char*>(p.ptsC + (long long)ntc * kTile * p.ldC16);
             issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
         }
-        slab_step(stage, more, gA, gB, offA, offB, 0);
+        slab_step(stage, more, gA, gB, offA, offB);
         stage ^= 1;
 
         if (kEpilogue) {
@@ -568,7 +575,30 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         tc = ntc;
         sumsBuf ^= 1;
     }
-    if (kEpilogue && staged > 0) flush_wave();
+    if (kEpilogue) {
+        // What is left in the eight regions goes out with one reservation for the workgroup: every workgroup
+        // ends at about the same time, and one atomic per wave, all on one address, would serialise for
+        // longer than a small join takes.  No transfer is in flight any more, so ordinary LDS accesses do.
+        unsigned* const sLeft = reinterpret_cast<unsigned*>(lds);  // the operand stages are free now
+        unsigned long long* const sBase = reinterpret_cast<unsigned long long*>(lds + 64);
+        const int ln = lane_now();
+        __syncthreads();  // every wave is past its last fragment read
+        if (ln == 0) sLeft[wave] = (unsigned)staged;
+        __syncthreads();
+        unsigned before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kThreads / 64; ++w) {
+            const unsigned left = __builtin_amdgcn_readfirstlane(sLeft[w]);
+            if (w < wave) before += left;
+            total += left;
+        }
+        if (total == 0) return;
+        if (wave == 0 && ln == 0) *sBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)total);
+        __syncthreads();
+        const unsigned long long base = *sBase + before;
+        for (int i = ln; i < staged; i += 64)
+            if (base + i < p.cap) p.pairs[base + i] = sStage[i];
+    }
 }
 
 }  // namespace

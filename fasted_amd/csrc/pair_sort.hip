@@ -65,28 +65,70 @@ unsigned grid_for(unsigned long long count) {
 
 }  // namespace
 
-hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream) {
-    if (count < 2) return hipSuccess;
-    auto* keys = static_cast<unsigned long long*>(pairs);
-    unsigned long long* alt = nullptr;
-    void* temp = nullptr;
-    size_t tempBytes = 0;
-    hipError_t e = hipMalloc(&alt, count * sizeof(unsigned long long));
-    if (e != hipSuccess) return e;
-    e = rocprim::radix_sort_keys(nullptr, tempBytes, keys, alt, (size_t)count, 0u, 64u, stream);
-    if (e == hipSuccess) e = hipMalloc(&temp, tempBytes ? tempBytes : 16);
-    if (e == hipSuccess) {
-        rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count);
-        e = rocprim::radix_sort_keys(temp, tempBytes, keys, alt, (size_t)count, 0u, 64u, stream);
-    }
-    if (e == hipSuccess) {
-        rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(alt, keys, count);
-        e = hipGetLastError();
-    }
-    hipError_t s = hipStreamSynchronize(stream);
-    if (e == hipSuccess) e = s;
+void SortBuffers::release() {
+    if (alt) (void)hipFree(alt);
     if (temp) (void)hipFree(temp);
-    (void)hipFree(alt);
+    alt = temp = nullptr;
+    altBytes = tempBytes = 0;
+}
+
+// Grows the two buffers of `ws` to what `count` records need; they are kept for the next sort.
+static hipError_t reserve_sort_buffers(SortBuffers* ws, unsigned long long count, hipStream_t stream) {
+    size_t needTemp = 0;
+    hipError_t e = rocprim::radix_sort_keys(nullptr, needTemp, static_cast<unsigned long long*>(nullptr),
+                                            static_cast<unsigned long long*>(nullptr), (size_t)count, 0u, 64u, stream);
+    if (e != hipSuccess) return e;
+    if (needTemp == 0) needTemp = 16;
+    const size_t needAlt = (size_t)count * sizeof(unsigned long long);
+    if (needAlt > ws->altBytes) {
+        if (ws->alt) (void)hipFree(ws->alt);
+        ws->alt = nullptr;
+        ws->altBytes = 0;
+        e = hipMalloc(&ws->alt, needAlt);
+        if (e != hipSuccess) return e;
+        ws->altBytes = needAlt;
+    }
+    if (needTemp > ws->tempBytes) {
+        if (ws->temp) (void)hipFree(ws->temp);
+        ws->temp = nullptr;
+        ws->tempBytes = 0;
+        e = hipMalloc(&ws->temp, needTemp);
+        if (e != hipSuccess) return e;
+        ws->tempBytes = needTemp;
+    }
+    return hipSuccess;
+}
+
+size_t sort_scratch_bytes(unsigned long long count) {
+    size_t needTemp = 0;
+    if (rocprim::radix_sort_keys(nullptr, needTemp, static_cast<unsigned long long*>(nullptr),
+                                 static_cast<unsigned long long*>(nullptr), (size_t)count, 0u, 64u, nullptr) != hipSuccess)
+        return 0;
+    return needTemp + (size_t)count * sizeof(unsigned long long);
+}
+
+hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws) {
+    if (count < 2) return hipSuccess;
+    SortBuffers local;
+    SortBuffers* const b = ws ? ws : &local;
+    hipError_t e = reserve_sort_buffers(b, count, stream);
+    auto* keys = static_cast<unsigned long long*>(pairs);
+    auto* alt = static_cast<unsigned long long*>(b->alt);
+    if (e == hipSuccess) {
+        size_t tempBytes = b->tempBytes;
+        rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count);
+        e = rocprim::radix_sort_keys(b->temp, tempBytes, keys, alt, (size_t)count, 0u, 64u, stream);
+        if (e == hipSuccess) {
+            rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(alt, keys, count);
+            e = hipGetLastError();
+        } else {
+            // the keys are still in place, rotated: put them back as they were
+            rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count);
+        }
+    }
+    const hipError_t s = hipStreamSynchronize(stream);
+    if (e == hipSuccess) e = s;
+    if (!ws) local.release();
     return e;
 }
 
