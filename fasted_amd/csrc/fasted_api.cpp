@@ -16,6 +16,7 @@
 #include <cstring>
 #include <fstream>
 #include <iostream>
+#include <memory>
 #include <string>
 #include <thread>
 #include <vector>
@@ -126,6 +127,8 @@ struct JoinScratch {
     hipEvent_t* ev;  // three events
 };
 
+fasted::SortBuffers g_sortWs;  // device buffers of the row-major sort, kept between calls
+
 // Three events around the two timed stages; created for the call, or borrowed from the caller.
 struct EventTimer {
     hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
@@ -176,7 +179,7 @@ struct PointSet {
 // are sorted outside the TFLOPS window.  `c.ptr == q.ptr` with selfJoin computes the norms once.
 void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon, void* dPairs,
                     unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats,
-                    const JoinScratch* fixed = nullptr) {
+                    const JoinScratch* fixed = nullptr, bool sortMayFail = false, int forcedStride = 0) {
     validate_shape(q.n, d, q.ld);
     validate_shape(c.n, d, c.ld);
     if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
@@ -224,6 +227,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.nQ = (int)q.n;
     jl.nC = (int)c.n;
     jl.selfJoin = selfJoin;
+    jl.forcedStride = forcedStride;
     jl.symmetric = selfJoin && (flags & FASTED_SYMMETRIC);
     jl.dPad = dPad;
     jl.halfQ = halfQ;
@@ -242,10 +246,19 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);
+    if (jl.symmetric) {
+        const unsigned long long side = ((unsigned long long)q.n + fasted::kTile - 1) / fasted::kTile;
+        cnt[2] = side * (side + 1) / 2;
+    }
     float sortMs = 0.f;
     if ((flags & FASTED_SORT_PAIRS) && cnt[1] > 1) {
         const auto w0 = std::chrono::steady_clock::now();
-        HIP_CHECK(fasted::sort_pairs_row_major(dPairs, cnt[1], stream));
+        const hipError_t e = fasted::sort_pairs_row_major(dPairs, cnt[1], stream, &g_sortWs);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            if (!sortMayFail) hip_check(e, "row-major sort of the pairs");
+            std::cout << "Failed to sort pairs: " << hipGetErrorString(e) << std::endl;
+        }
         sortMs = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
     }
     if (stats) {
@@ -420,7 +433,7 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
             before = after;
         }
         const unsigned long long kept = std::min(before, devCap);
-        if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute));
+        if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute, &g_sortWs));
         HIP_CHECK(hipStreamSynchronize(dev.compute));
         const unsigned long long take = std::min(kept, cap - storedAll);
         if (take)
@@ -474,50 +487,140 @@ char* write_index(char* end, int value) {
 
 // "q, c\n" per pair, the format of operator<< in source/pair.cuh:51-54; with distances
 // "q, c, dist\n", the three-column form results/scripts/neighbor_tables.py:102-115 also reads.
-// The lines are formatted by several threads, a slice of the list each, into buffers that are then
-// written in order (one formatted-print call per pair made large lists take minutes).
-void write_pairs_text(const std::string& path, const std::vector<FastedPair>& pairs, const std::vector<float>& dist) {
-    std::FILE* f = std::fopen(path.c_str(), "w");
-    if (!f) throw std::ios_base::failure("Failed to open output file: " + path);
-    const bool withDistance = dist.size() == pairs.size() && !pairs.empty();
-    const size_t chunk = 1u << 20;  // pairs per buffer
-    const unsigned threads = std::max(1u, std::min(fasted::host_threads("FASTED_CSV_THREADS"),
-                                                   static_cast<unsigned>((pairs.size() + chunk - 1) / chunk)));
-    std::vector<std::string> text(threads);
-    bool failed = false;
-    for (size_t base = 0; base < pairs.size() && !failed; base += chunk * threads) {
-        auto format = [&](unsigned w) {
-            const size_t lo = std::min(pairs.size(), base + w * chunk), hi = std::min(pairs.size(), lo + chunk);
-            std::string& out = text[w];
-            out.clear();
-            out.reserve((hi - lo) * (withDistance ? 40 : 24));
-            char line[64];
-            for (size_t i = lo; i < hi; ++i) {
-                char* end = line + sizeof line;
-                *--end = '\n';
-                if (withDistance) {
-                    char number[32];
-                    const int len = std::snprintf(number, sizeof number, "%.7g", dist[i]);
-                    end -= len;
-                    std::memcpy(end, number, static_cast<size_t>(len));
+// Pairs arrive in pieces (the download of the next piece runs while this one is written).  The lines of a
+// piece are formatted by several threads, a slice each, into buffers that are then written in order (one
+// formatted-print call per pair made large lists take minutes).
+class PairsTextFile {
+public:
+    explicit PairsTextFile(const std::string& path) : path_(path), f_(std::fopen(path.c_str(), "w")) {
+        if (!f_) throw std::ios_base::failure("Failed to open output file: " + path);
+    }
+    PairsTextFile(const PairsTextFile&) = delete;
+    PairsTextFile& operator=(const PairsTextFile&) = delete;
+    ~PairsTextFile() {
+        if (f_) (void)std::fclose(f_);
+    }
+    // `dist` may be null: two columns
+    void append(const FastedPair* pairs, const float* dist, size_t count) {
+        const size_t slice = 1u << 20;  // pairs per buffer
+        const unsigned threads = std::max(1u, std::min(fasted::host_threads("FASTED_CSV_THREADS"),
+                                                       static_cast<unsigned>((count + slice - 1) / slice)));
+        text_.resize(std::max<size_t>(text_.size(), threads));
+        for (size_t base = 0; base < count && !failed_; base += slice * threads) {
+            auto format = [&](unsigned w) {
+                const size_t lo = std::min(count, base + w * slice), hi = std::min(count, lo + slice);
+                std::string& out = text_[w];
+                out.clear();
+                out.reserve((hi - lo) * (dist ? 40 : 24));
+                char line[64];
+                for (size_t i = lo; i < hi; ++i) {
+                    char* end = line + sizeof line;
+                    *--end = '\n';
+                    if (dist) {
+                        char number[32];
+                        const int len = std::snprintf(number, sizeof number, "%.7g", dist[i]);
+                        end -= len;
+                        std::memcpy(end, number, static_cast<size_t>(len));
+                        *--end = ' ';
+                        *--end = ',';
+                    }
+                    end = write_index(end, pairs[i].CandidatePoint);
                     *--end = ' ';
                     *--end = ',';
+                    end = write_index(end, pairs[i].QueryPoint);
+                    out.append(end, static_cast<size_t>(line + sizeof line - end));
                 }
-                end = write_index(end, pairs[i].CandidatePoint);
-                *--end = ' ';
-                *--end = ',';
-                end = write_index(end, pairs[i].QueryPoint);
-                out.append(end, static_cast<size_t>(line + sizeof line - end));
-            }
-        };
-        std::vector<std::thread> pool;
-        for (unsigned w = 1; w < threads; ++w) pool.emplace_back(format, w);
-        format(0);
-        for (auto& t : pool) t.join();
-        for (unsigned w = 0; w < threads && !failed; ++w)
-            if (!text[w].empty() && std::fwrite(text[w].data(), 1, text[w].size(), f) != text[w].size()) failed = true;
+            };
+            std::vector<std::thread> pool;
+            for (unsigned w = 1; w < threads; ++w) pool.emplace_back(format, w);
+            format(0);
+            for (auto& t : pool) t.join();
+            for (unsigned w = 0; w < threads && !failed_; ++w)
+                if (!text_[w].empty() && std::fwrite(text_[w].data(), 1, text_[w].size(), f_) != text_[w].size())
+                    failed_ = true;
+        }
     }
-    if (std::fclose(f) != 0 || failed) throw std::ios_base::failure("Failed to write output file: " + path);
+    void close() {
+        const bool bad = std::fclose(f_) != 0 || failed_;
+        f_ = nullptr;
+        if (bad) throw std::ios_base::failure("Failed to write output file: " + path_);
+    }
+
+private:
+    std::string path_;
+    std::FILE* f_;
+    std::vector<std::string> text_;
+    bool failed_ = false;
+};
+
+// Device and pinned host memory of the drop-in entry points that outlives a call: the pair buffer, the
+// distance column, and two pinned pieces through which the sorted pairs leave the device.  reRun() on a
+// resident dataset allocates nothing.
+struct PairWorkspace {
+    void* dPairs = nullptr;
+    unsigned long long capPairs = 0;
+    float* dDist = nullptr;
+    unsigned long long capDist = 0;
+    static constexpr size_t kPiecePairs = (size_t)4 << 20;  // 32 MiB of records per piece
+    FastedPair* hPairs[2] = {nullptr, nullptr};
+    float* hDist[2] = {nullptr, nullptr};
+    hipEvent_t landed[2] = {nullptr, nullptr};
+    hipStream_t copy = nullptr;
+
+    void ensure_host() {
+        if (copy) return;
+        HIP_CHECK(hipStreamCreateWithFlags(&copy, hipStreamNonBlocking));  // default priority
+        for (int i = 0; i < 2; ++i) {
+            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hPairs[i]), kPiecePairs * sizeof(FastedPair), hipHostMallocDefault));
+            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hDist[i]), kPiecePairs * sizeof(float), hipHostMallocDefault));
+            HIP_CHECK(hipEventCreateWithFlags(&landed[i], hipEventDisableTiming));
+        }
+    }
+    void release() {
+        if (dPairs) (void)hipFree(dPairs);
+        if (dDist) (void)hipFree(dDist);
+        dPairs = nullptr;
+        dDist = nullptr;
+        capPairs = capDist = 0;
+        for (int i = 0; i < 2; ++i) {
+            if (hPairs[i]) (void)hipHostFree(hPairs[i]);
+            if (hDist[i]) (void)hipHostFree(hDist[i]);
+            if (landed[i]) (void)hipEventDestroy(landed[i]);
+            hPairs[i] = nullptr;
+            hDist[i] = nullptr;
+            landed[i] = nullptr;
+        }
+        if (copy) (void)hipStreamDestroy(copy);
+        copy = nullptr;
+    }
+} g_pairWs;
+
+// Pair buffer of N*256 records (source/findPairs.cuh:644-647), shrunk to what the device can hold together
+// with what the sort of a full buffer needs (a second key buffer and the radix sort's storage), as
+// Pairs::init shrinks it to the free memory (source/pair.cuh:69-85).  Kept until a larger one is needed.
+unsigned long long ensure_pair_buffer(int n) {
+    const unsigned long long want = (unsigned long long)n * 256ull;
+    if (g_pairWs.dPairs && g_pairWs.capPairs >= want) return want;
+    if (g_pairWs.dPairs) {
+        HIP_CHECK(hipFree(g_pairWs.dPairs));
+        g_pairWs.dPairs = nullptr;
+        g_pairWs.capPairs = 0;
+    }
+    g_sortWs.release();
+    size_t freeB = 0, totalB = 0;
+    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
+    const size_t usable = freeB - freeB / 16;  // leave some room for the runtime
+    unsigned long long maxPairs = want;
+    for (int round = 0; round < 4; ++round) {
+        const size_t need = (size_t)maxPairs * sizeof(FastedPair) + fasted::sort_scratch_bytes(maxPairs);
+        if (need <= usable) break;
+        maxPairs = (unsigned long long)((double)maxPairs * (double)usable / (double)need * 0.98);
+    }
+    if (maxPairs < want)
+        std::printf("Failed to allocate enough space for %llu pairs. Reducing max number of pairs to %llu\n", want, maxPairs);
+    HIP_CHECK(hipMalloc(&g_pairWs.dPairs, (size_t)(maxPairs ? maxPairs : 1) * sizeof(FastedPair)));
+    g_pairWs.capPairs = maxPairs;
+    return maxPairs;
 }
 
 Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, const std::string& datasetName) {
@@ -535,56 +638,63 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
     }
     HIP_CHECK(hipDeviceSynchronize());
 
-    // Pair buffer: N*256 records, shrunk to what the device can still hold
-    // (source/findPairs.cuh:644-647, source/pair.cuh:69-85).  Half of the free memory is the
-    // limit here because the row-major sort needs a second buffer of the stored size.
-    unsigned long long maxPairs = (unsigned long long)tb.n * 256ull;
-    size_t freeB = 0, totalB = 0;
-    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
-    const unsigned long long fit = (unsigned long long)(freeB / 2) / sizeof(FastedPair);
-    if (maxPairs > fit) {
-        std::printf("Failed to allocate enough space for %llu pairs. Reducing max number of pairs to %llu\n", maxPairs,
-                    fit);
-        maxPairs = fit;
-    }
-    void* dPairs = nullptr;
-    HIP_CHECK(hipMalloc(&dPairs, (size_t)(maxPairs ? maxPairs : 1) * sizeof(FastedPair)));
+    const unsigned long long maxPairs = std::min(ensure_pair_buffer(tb.n), g_pairWs.capPairs);
+    g_pairWs.ensure_host();
+    void* const dPairs = g_pairWs.dPairs;
 
     FastedJoinStats st{};
-    std::vector<FastedPair> pairs;
-    std::vector<float> distances;
-    try {
-        const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
-        join_on_device(all, all, true, tb.dPad, epsilon, dPairs, maxPairs, FASTED_SORT_PAIRS, nullptr, &st);
-        if (!quiet()) {
-            std::printf("Number of pairs found %llu\n", st.pairsFound);
-            std::printf("Number of pairs stored %llu\n", st.pairsStored);
-        }
-        // the pairs always leave the device, saved or not (source/findPairs.cuh:705-714)
-        pairs.resize((size_t)st.pairsStored);
-        if (st.pairsStored)
-            HIP_CHECK(hipMemcpy(pairs.data(), dPairs, pairs.size() * sizeof(FastedPair), hipMemcpyDeviceToHost));
-        if (savePairs && save_distances() && st.pairsStored) {
-            float* dDist = nullptr;
-            HIP_CHECK(hipMalloc(&dDist, pairs.size() * sizeof(float)));
-            hipError_t e = fasted::launch_pair_distances(g_res.dPoints, tb.dPad, tb.n, g_res.dPoints, tb.dPad, tb.n,
-                                                         tb.dPad, dPairs, st.pairsStored, dDist, nullptr);
-            distances.resize(pairs.size());
-            if (e == hipSuccess)
-                e = hipMemcpy(distances.data(), dDist, distances.size() * sizeof(float), hipMemcpyDeviceToHost);
-            (void)hipFree(dDist);
-            HIP_CHECK(e);
-        }
-    } catch (...) {
-        (void)hipFree(dPairs);
-        throw;
+    const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
+    // a sort that fails (no memory for its buffers) is reported and the pairs leave unsorted, as the
+    // reference carries on after "Failed to sort pairs" (source/findPairs.cuh:701-718)
+    join_on_device(all, all, true, tb.dPad, epsilon, dPairs, maxPairs, FASTED_SORT_PAIRS, nullptr, &st, nullptr,
+                   /*sortMayFail=*/true);
+    if (!quiet()) {
+        std::printf("Number of pairs found %llu\n", st.pairsFound);
+        std::printf("Number of pairs stored %llu\n", st.pairsStored);
     }
-    HIP_CHECK(hipFree(dPairs));
+    const bool withDistance = savePairs && save_distances() && st.pairsStored > 0;
+    if (withDistance) {
+        if (g_pairWs.capDist < st.pairsStored) {
+            if (g_pairWs.dDist) HIP_CHECK(hipFree(g_pairWs.dDist));
+            g_pairWs.dDist = nullptr;
+            g_pairWs.capDist = 0;
+            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_pairWs.dDist), (size_t)st.pairsStored * sizeof(float)));
+            g_pairWs.capDist = st.pairsStored;
+        }
+        HIP_CHECK(fasted::launch_pair_distances(g_res.dPoints, tb.dPad, tb.n, g_res.dPoints, tb.dPad, tb.n, tb.dPad, dPairs,
+                                                st.pairsStored, g_pairWs.dDist, nullptr));
+        HIP_CHECK(hipStreamSynchronize(nullptr));
+    }
+
+    // The pairs always leave the device, saved or not (source/findPairs.cuh:705-714): piece by piece through
+    // two pinned buffers, the next piece travelling while the current one is written as text.
+    std::unique_ptr<PairsTextFile> file;
     if (savePairs) {
         const std::string path = output_dir() + "/" + datasetName + "_" + std::to_string(epsilon) + ".pairs";
         std::cout << "Output file is: " << path << std::endl;
-        write_pairs_text(path, pairs, distances);
+        file.reset(new PairsTextFile(path));
     }
+    const size_t piece = PairWorkspace::kPiecePairs;
+    const size_t total = (size_t)st.pairsStored;
+    auto fetch = [&](size_t first, int slot) {
+        const size_t count = std::min(piece, total - first);
+        HIP_CHECK(hipMemcpyAsync(g_pairWs.hPairs[slot], static_cast<const FastedPair*>(dPairs) + first,
+                                 count * sizeof(FastedPair), hipMemcpyDeviceToHost, g_pairWs.copy));
+        if (withDistance)
+            HIP_CHECK(hipMemcpyAsync(g_pairWs.hDist[slot], g_pairWs.dDist + first, count * sizeof(float),
+                                     hipMemcpyDeviceToHost, g_pairWs.copy));
+        HIP_CHECK(hipEventRecord(g_pairWs.landed[slot], g_pairWs.copy));
+    };
+    if (total) fetch(0, 0);
+    int slot = 0;
+    for (size_t first = 0; first < total; first += piece, slot ^= 1) {
+        HIP_CHECK(hipEventSynchronize(g_pairWs.landed[slot]));
+        if (first + piece < total) fetch(first + piece, slot ^ 1);
+        if (file) file->append(g_pairWs.hPairs[slot], withDistance ? g_pairWs.hDist[slot] : nullptr, std::min(piece, total - first));
+    }
+    if (file) file->close();
+
+    // the reference's total also spans the writing of the file (source/findPairs.cuh:700-726)
     const double totalTime = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
     const float kernelSec = (st.sumSquaredMs + st.joinMs) / 1000.0f;
     // unpadded shape: padded zeros are not useful work (source/findPairs.cuh:745-747)
@@ -674,7 +784,9 @@ FastedJoinStats count_resident(double epsilon) {
 }
 
 // Count-only join of an evenly spaced sample of the resident points against all of them.  Every sampled
-// point meets itself among the candidates, so found - sampleRows estimates sampleRows x selectivity.
+// point meets itself among the candidates -- that pair is forced like the self pairs of the full join, so the
+// sampled and the full count treat a point's own pair alike -- and found - sampleRows estimates
+// sampleRows x selectivity.
 FastedJoinStats count_resident_sampled(double epsilon, int sampleRows) {
     ensure_resident_uploaded();
     const fasted::PointTable& tb = g_res.table;
@@ -694,7 +806,8 @@ FastedJoinStats count_resident_sampled(double epsilon, int sampleRows) {
     FastedJoinStats st{};
     const PointSet sample{g_res.dSample, sampleRows, tb.dPad, nullptr};
     const PointSet all{g_res.dPoints, tb.n, tb.dPad, nullptr};
-    join_on_device(sample, all, false, tb.dPad, epsilon, nullptr, 0, 0, nullptr, &st);
+    join_on_device(sample, all, false, tb.dPad, epsilon, nullptr, 0, 0, nullptr, &st, nullptr, false,
+                   /*forcedStride=*/tb.n / sampleRows);
     return st;
 }
 
@@ -778,6 +891,8 @@ void releaseResources(void) {
     g_res.drop_device();
     g_res.table = fasted::PointTable();
     g_ws.release();
+    g_pairWs.release();
+    g_sortWs.release();
 }
 
 int fasted_self_join_device(const void* d_points, long long n, int d, long long ld, double epsilon, float* d_sums,
@@ -834,6 +949,21 @@ int fasted_pair_distances_device(const void* d_queries, long long n_queries, lon
                                                 (int)n_candidates, round_up(d, fasted::kSlabK), d_pairs, count,
                                                 d_distances, static_cast<hipStream_t>(stream)));
         HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    });
+}
+
+int fasted_check_padding_device(const void* d_points, long long n, int d, long long ld, unsigned long long* bad_rows,
+                                void* stream) {
+    return guarded([&] {
+        if (!d_points || !bad_rows) throw std::invalid_argument("null pointer");
+        validate_shape(n, d, ld);
+        g_ws.ensure(1);
+        unsigned long long* const word = g_ws.counters;  // word 0 of the counter block is free between joins
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, s));
+        HIP_CHECK(fasted::launch_padding_check(d_points, ld, (int)n, d, round_up(d, fasted::kSlabK), word, s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        HIP_CHECK(hipMemcpy(bad_rows, word, sizeof *bad_rows, hipMemcpyDeviceToHost));
     });
 }
 

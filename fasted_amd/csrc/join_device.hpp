@@ -24,7 +24,7 @@ struct JoinParams {
     const u32x4* ptsC;  // candidate rows (the same buffer for a self-join)
     long long ldQ16, ldC16;  // row strides in 16-byte units
     int nQ, nC;
-    int selfJoin;  // queries and candidates are the same set: (i, i) is always a pair
+    int selfStride;  // != 0: (q, q * selfStride) is always a pair -- 1 for a self-join ((i, i) is a pair)
     int symmetric; // self-join only: compute tiles on and above the diagonal, emit (q,c) and (c,q)
     int nSlabs;    // 64-wide k-slabs per tile
     const float* halfQ;  // per query point: eps^2/4 - s/2, s = squared norm

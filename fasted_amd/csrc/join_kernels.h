@@ -16,6 +16,8 @@ struct JoinLaunch {
     long long ldQ, ldC;          // row strides in halves (multiples of 8)
     int nQ, nC;                  // real points
     bool selfJoin;               // same set on both sides: (i, i) always counts as a pair
+    int forcedStride = 0;        // two sets where query i IS candidate i * forcedStride (a sample of the
+                                 // candidates joined against all of them): that pair always counts
     bool symmetric;              // self-join: only tiles on/above the diagonal are computed, pairs mirrored
     int dPad;                    // K extent, multiple of kSlabK
     const float* halfQ;          // per query point: eps^2/4 - s/2 (s = squared norm), see launch_sum_squared
@@ -44,6 +46,9 @@ hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad,
 // The same halves from norms that are already there.
 hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, unsigned long long* counters,
                          hipStream_t stream);
+// *badRows += number of rows whose columns d .. dPad-1 are not all zeros.
+hipError_t launch_padding_check(const void* points, long long ld, int n, int d, int dPad, unsigned long long* badRows,
+                                hipStream_t stream);
 // Clears the queue heads and, unless keepFound, the pair counter and the non-finite flag (words 0, 1 of `counters`).
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream);
 // pairs[first, last): QueryPoint += qOffset, CandidatePoint += cOffset.

@@ -135,6 +135,18 @@ __global__ void __launch_bounds__(256) halves_kernel(const float* __restrict__ s
     if (!(__builtin_fabsf(s) < __builtin_inff())) counters[kCounterNonFinite] = 1ull;
 }
 
+// Rows whose padding columns d .. dPad-1 hold anything but zeros (the kernels read them unmasked, so they must
+// be zeros: a caller's mistake that would otherwise show up as silently wrong norms and pairs).
+__global__ void __launch_bounds__(256) padding_check_kernel(const unsigned short* __restrict__ pts, long long ld, int n, int d,
+                                                            int dPad, unsigned long long* __restrict__ badRows) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n) return;
+    const unsigned short* p = pts + (long long)row * ld;
+    bool bad = false;
+    for (int k = d; k < dPad; ++k) bad |= (p[k] & 0x7fffu) != 0u;  // +0 and -0 are both fine
+    if (bad) atomicAdd(badRows, 1ull);
+}
+
 // Clears the queue heads and, unless `keepFound`, the pair counter (word 0) and the non-finite flag (word 1):
 // a launch that keeps them appends its pairs behind those of the launch before.
 __global__ void reset_counters_kernel(unsigned long long* c, int keepFound) {
@@ -455,7 +467,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             // Every element is tested one by one when the tile touches the diagonal of a self-join or the ragged
             // end of a dataset (self pairs are forced, padded rows/columns masked: source/warpMma.cuh:257-259)
             // or when the dataset holds points with non-finite norms (a NaN must compare as "no hit").
-            const bool edge = nonFinite || (p.selfJoin && tr == tc) || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
+            // (forced pairs: query q with candidate q * selfStride -- the diagonal of a self-join, or the sampled
+            // points among all points)
+            const bool diagonal = p.selfStride != 0 && colBase <= (rowBase + kTile - 1) * p.selfStride &&
+                                  rowBase * p.selfStride <= colBase + kTile - 1;
+            const bool edge = nonFinite || diagonal || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
             const bool mirror = p.symmetric && tr != tc;  // a tile above the diagonal also stands for its mirror image
 
             // Per-lane hit bits of the 4 pairs of block rows: element e = (fi & 1) * 16 + fj * 4 + r of the pair
@@ -517,7 +533,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                             for (int r = 0; r < 4; ++r) {
                                 const int q = qLane + fi * 16 + r, c = cLane + fj * 16;
                                 const bool hit =
-                                    ((acc[fi][fj][r] >= 0.0f) | ((p.selfJoin != 0) & (q == c))) & (q < p.nQ) & (c < p.nC);
+                                    ((acc[fi][fj][r] >= 0.0f) | ((p.selfStride != 0) & (q * p.selfStride == c))) & (q < p.nQ) & (c < p.nC);
                                 m = (m << 1) | (hit ? 1u : 0u);
                             }
                         }
@@ -653,6 +669,14 @@ hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, un
     return hipGetLastError();
 }
 
+hipError_t launch_padding_check(const void* points, long long ld, int n, int d, int dPad, unsigned long long* badRows,
+                                hipStream_t stream) {
+    if (dPad > d)
+        padding_check_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(
+            static_cast<const unsigned short*>(points), ld, n, d, dPad, badRows);
+    return hipGetLastError();
+}
+
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream) {
     reset_counters_kernel<<<1, 256, 0, stream>>>(counters, keepFound ? 1 : 0);
     return hipGetLastError();
@@ -688,7 +712,7 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     p.ldC16 = l.ldC / 8;
     p.nQ = l.nQ;
     p.nC = l.nC;
-    p.selfJoin = l.selfJoin ? 1 : 0;
+    p.selfStride = l.forcedStride > 0 ? l.forcedStride : (l.selfJoin ? 1 : 0);
     p.symmetric = (l.selfJoin && l.symmetric) ? 1 : 0;
     p.nSlabs = l.dPad / kSlabK;
     p.halfQ = l.halfQ;

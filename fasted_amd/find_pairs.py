@@ -136,6 +136,9 @@ def load_findpairs(path: str = None):
     lib.fasted_find_epsilon_sampled.restype = c.c_int
     lib.fasted_find_epsilon_sampled.argtypes = [c.c_double, c.c_double, c.c_int, c.POINTER(c.c_double),
                                                 c.POINTER(c.c_double), c.POINTER(c.c_int)]
+    lib.fasted_check_padding_device.restype = c.c_int
+    lib.fasted_check_padding_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong,
+                                                c.POINTER(c.c_ulonglong), c.c_void_p]
     lib.fasted_sum_squared_device.restype = c.c_int
     lib.fasted_sum_squared_device.argtypes = [c.c_void_p, c.c_longlong, c.c_int, c.c_longlong, c.c_void_p, c.c_void_p]
     lib.fasted_raster_coord.restype = c.c_int
@@ -289,6 +292,14 @@ def join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates
     _check(lib, lib.fasted_join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates,
                                        d, float(epsilon), None, None, pairs_ptr, cap, flags, stream, ctypes.byref(st)))
     return st
+
+
+def check_padding_device(points_ptr, n, d, ld, stream=None):
+    """Rows whose padding columns d..roundup(d,64) are not all zeros (must be 0 for the device entries)."""
+    lib = load_findpairs()
+    bad = ctypes.c_ulonglong()
+    _check(lib, lib.fasted_check_padding_device(points_ptr, n, d, ld, ctypes.byref(bad), stream))
+    return bad.value
 
 
 def sum_squared_device(points_ptr, n, d, ld, sums_ptr, stream=None):

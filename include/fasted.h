@@ -34,8 +34,11 @@ typedef struct mmaShape {
 
 /* source/findPairs.cuh:37-46; mirrored by find_pairs.py:24-44.  56 bytes. */
 typedef struct Results {
-    double totalTime;              /* seconds: upload + kernels + sort + download, no disk */
-    double TFLOPS;                 /* 2*N*N*D / (sumSquared + join kernel time) / 1e12, unpadded N, D */
+    double totalTime;              /* seconds: upload + kernels + sort + download and, with savePairs, the writing of
+                                      the .pairs file (as source/findPairs.cuh:700-726 times it) */
+    double TFLOPS;                 /* 2*N*N*D / (counter reset + sumSquared + join kernel time) / 1e12, unpadded N, D.
+                                      The reference's window (source/findPairs.cuh:625-697,729) also spans its pair-buffer
+                                      allocation and rasterizer set-up; here the pair buffer is kept between calls */
     unsigned long long pairsFound; /* every ordered pair with dist <= eps, self pairs included */
     unsigned long long pairsStored; /* <= pairsFound when the pair buffer overflowed */
     mmaShape inputProblemShape;    /* (N, N, D) as given */
@@ -68,12 +71,12 @@ void releaseResources(void);
  * Return 0 on success, non-zero on failure; fasted_last_error() then describes it.     */
 
 typedef struct FastedJoinStats {
-    float sumSquaredMs; /* HIP-event time of the squared-norm pre-pass */
-    float joinMs;       /* HIP-event time of counter reset + join kernel */
-    float sortMs;       /* HIP-event time of the row-major sort (0 when not sorted) */
+    float sumSquaredMs; /* HIP-event time of counter reset + squared-norm pre-pass */
+    float joinMs;       /* HIP-event time of the join kernel */
+    float sortMs;       /* host wall time of the row-major sort, stream synchronisation included (0 when not sorted) */
     int paddedN;        /* rows covered by the tile grid */
     int paddedD;        /* K extent the kernel looped over */
-    unsigned long long tiles;      /* non-empty 256x256 tiles processed */
+    unsigned long long tiles;      /* 256x256 tiles computed (with FASTED_SYMMETRIC: those on and above the diagonal) */
     unsigned long long pairsFound;
     unsigned long long pairsStored;
 } FastedJoinStats;
@@ -157,6 +160,14 @@ int fasted_join_device(const void* d_queries, long long n_queries, long long ld_
 int fasted_pair_distances_device(const void* d_queries, long long n_queries, long long ld_queries,
                                  const void* d_candidates, long long n_candidates, long long ld_candidates, int d,
                                  const FastedPair* d_pairs, unsigned long long count, float* d_distances, void* stream);
+
+/* Checks the one precondition of the device entries that they cannot see for themselves: with D % 64 != 0 the
+ * columns D .. roundup(D,64)-1 of every row must be zeros (the kernels read whole 64-wide slabs unmasked, as the
+ * reference reads its zero padding, source/DataLoader/PointListBuilder.hpp:149-179).  *bad_rows = number of rows
+ * that hold anything else there (0 = fine; always 0 when D % 64 == 0).  No counterpart in the reference, whose
+ * only data path pads on the host. */
+int fasted_check_padding_device(const void* d_points, long long n, int d, long long ld, unsigned long long* bad_rows,
+                                void* stream);
 
 /* Squared norms only: sums[i] = sum_k x_ik^2 in FP32.  Replaces
  * SumSqd::ComputeSquaredSums (source/sumSquared.cuh:84-118). */

@@ -195,3 +195,63 @@ def test_pairs_file_with_the_distance_column(lib, tmp_path):
     assert (dist <= eps * (1 + 1e-3)).all()
     lib.releaseResources()
     lib.fasted_set_output_dir(b"")
+
+
+def test_large_pair_list_leaves_the_device_in_pieces(lib, tmp_path):
+    """More stored pairs than one download piece holds (4 Mi records): the .pairs file must still be the whole
+    sorted list, with and without the distance column, and a second reRun (which reuses the pair buffer, the
+    sort buffers and the pinned pieces) must write the same bytes."""
+    import torch
+
+    import fasted_amd
+
+    n, d = 20000, 64  # the pair buffer holds N*256 records: 230 neighbours per point fit, in two pieces
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    bits, n_, d_, name = fasted_amd.resident_points()
+    eps = datasets.epsilon_for_neighbours(bits[:n, :d], 230)
+    lib.fasted_set_output_dir(str(tmp_path).encode())
+    r = lib.reRun(eps, True)
+    assert r.pairsStored == r.pairsFound > 4 * (1 << 20)
+    path = tmp_path / ("%s_%f.pairs" % (name, eps))
+    first = path.read_bytes()
+    got = np.loadtxt(path, delimiter=",", dtype=np.int64)
+    assert got.shape == (r.pairsStored, 2)
+    key = got[:, 0] * n + got[:, 1]
+    assert np.all(key[1:] > key[:-1])  # row-major, no duplicates, across the piece boundaries too
+    # the same list through the device entry
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    cap = int(r.pairsStored) + 1024
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    st = fasted_amd.self_join_device(pts.data_ptr(), n, d, bits.shape[1], eps, pairs.data_ptr(), cap)
+    assert st.pairsStored == r.pairsStored
+    assert np.array_equal(pairs[: st.pairsStored].cpu().numpy().astype(np.int64), got)
+    # again: nothing is allocated this time, the bytes are the same
+    r2 = lib.reRun(eps, True)
+    assert r2.pairsStored == r.pairsStored and path.read_bytes() == first
+    # with the distance column
+    lib.fasted_set_save_distances(1)
+    r3 = lib.reRun(eps, True)
+    lib.fasted_set_save_distances(0)
+    with open(path) as f:
+        head = [next(f) for _ in range(3)]
+    assert all(re.fullmatch(r"\d+, \d+, [0-9.e+-]+\n", line) for line in head)
+    with open(path) as f:
+        assert sum(1 for _ in f) == r3.pairsStored
+    lib.releaseResources()
+    lib.fasted_set_output_dir(b"")
+
+
+def test_sampled_probe_counts_a_points_own_pair_like_the_full_count(lib):
+    """At a tiny epsilon only the self pairs remain: the sampled probe (sample x all points) must report
+    exactly its sampled rows, as the full count reports exactly N -- large norms included, where the
+    expansion s_q + s_c - 2 q.c alone would lose some of them."""
+    import ctypes
+
+    n, d = 6000, 512
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    found, rows, secs = ctypes.c_ulonglong(), ctypes.c_int(), ctypes.c_double()
+    assert lib.fasted_count_pairs(1e-4, ctypes.byref(found), ctypes.byref(secs)) == 0
+    assert found.value == n
+    assert lib.fasted_count_pairs_sampled(1e-4, 1000, ctypes.byref(found), ctypes.byref(rows), ctypes.byref(secs)) == 0
+    assert rows.value == 1000 and found.value == 1000
+    lib.releaseResources()

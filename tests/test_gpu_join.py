@@ -340,3 +340,59 @@ def test_points_with_infinite_coordinates_pair_with_nothing_but_themselves(faste
     keep = ~(np.isin(clean[:, 0], odd) | np.isin(clean[:, 1], odd))
     want = oracle.sort_pairs(np.vstack([clean[keep], [[i, i] for i in odd]]).astype(np.int32))
     assert np.array_equal(got, want)
+
+
+def test_padding_columns_are_checked(fasted):
+    """D % 64 != 0: the device entries read whole 64-wide slabs, so the padding columns must be zeros;
+    fasted_check_padding_device counts the rows where they are not."""
+    import torch
+
+    n, d, ld = 700, 40, 64
+    bits = np.zeros((n, ld), dtype=np.uint16)
+    bits[:, :d] = datasets.exponential(n, d, seed=3)
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    assert fasted.check_padding_device(pts.data_ptr(), n, d, ld) == 0
+    bits[5, 41] = 0x3C00   # 1.0 in a padding column
+    bits[699, 63] = 0x0001  # the smallest subnormal
+    bits[9, 50] = 0x8000   # -0.0 is as good as zero
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    assert fasted.check_padding_device(pts.data_ptr(), n, d, ld) == 2
+    assert fasted.check_padding_device(pts.data_ptr(), n, 64, ld) == 0  # no padding columns at all
+
+
+def test_join_is_deterministic_over_many_tiles_per_workgroup(fasted):
+    """Every workgroup walks hundreds of tiles here, with the next tile's operands in flight during each
+    epilogue: two runs must give the same pair set (a transfer that a barrier did not wait for shows up as a
+    few pairs that differ from run to run), and sampled rows must agree with FP64."""
+    import torch
+
+    n, d = 90000, 192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+    centers = torch.rand((300, d), generator=g, device="cuda")
+    which = torch.randint(0, 300, (n,), generator=g, device="cuda")
+    pts = (centers[which] + 0.05 * torch.randn((n, d), generator=g, device="cuda")).to(torch.float16)
+    x = pts[:2048].double()
+    d2 = ((x * x).sum(1)[:, None] + (x * x).sum(1)[None, :] - 2.0 * x @ x.T)
+    eps = float(torch.quantile(d2[d2 > 1e-6].flatten()[:1 << 20], 0.004).sqrt())
+    cap = 400 * n
+    keys = []
+    for _ in range(2):
+        pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+        st = fasted.self_join_device(pts.view(torch.int16).data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, flags=0)
+        assert st.pairsFound == st.pairsStored > 10 * n
+        got = pairs[: st.pairsStored]
+        keys.append(torch.sort(got[:, 0].to(torch.int64) * n + got[:, 1].to(torch.int64)).values)
+        del pairs
+    assert keys[0].shape == keys[1].shape and bool((keys[0] == keys[1]).all())
+    rows = torch.arange(0, n, n // 256, device="cuda")[:256]
+    xs = pts[rows].double()
+    d2 = ((xs * xs).sum(1)[:, None] + (pts.double() ** 2).sum(1)[None, :] - 2.0 * xs @ pts.double().T).clamp_min(0)
+    truth = d2 <= eps * eps
+    mask = torch.zeros_like(truth)
+    q, c = keys[0] // n, keys[0] % n
+    sel = torch.isin(q, rows)
+    mask[torch.searchsorted(rows, q[sel]), c[sel]] = True
+    diff = truth != mask
+    rel = (d2[diff].sqrt() - eps).abs() / eps
+    assert int((rel > 1e-3).sum()) == 0, (int(diff.sum()), float(rel.max()))
