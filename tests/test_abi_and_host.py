@@ -256,8 +256,10 @@ class MockFindPairs:
         return fp.compute_selectivity(found, self.n)
 
 
-def test_epsilon_search_follows_the_reference_procedure():
-    from fasted_amd import experiments as ex
+def test_epsilon_search_restatement_follows_the_reference_procedure():
+    """The checker's restatement of the reference's search (oracle/epsilon_search.py) against what the
+    procedure fixes on a closed-form selectivity: the exact sequence of probes."""
+    from oracle import epsilon_search as ex
 
     assert ex.within_percent(100.5, 100, 0.01) and not ex.within_percent(102, 100, 0.01)
     assert ex.adjust_epsilon_binary(4.0, 8.0, 64, 100) == 2.0  # overshoot: half a step back
@@ -274,10 +276,14 @@ def test_epsilon_search_follows_the_reference_procedure():
     eps = ex.find_epsilon_binary(64, mock.selectivity)
     assert ex.within_percent(700.0 * eps ** 3, 64, 0.011)
     assert mock.calls[:2] == [2.0, 1.0]  # the upper bound, then the midpoint of (0, 2)
+    # selectivity = 1000 eps: target 250 is hit exactly by the probes 2 (bound), 1, 0.5, 0.25
+    calls = []
+    assert ex.find_epsilon_binary(250, lambda e: calls.append(e) or 1000.0 * e) == 0.25
+    assert calls == [2.0, 1.0, 0.5, 0.25]
 
 
 def test_pair_statistics_and_per_point_iou():
-    from fasted_amd import experiments as ex
+    from fasted_amd import accuracy as ex
 
     five = np.array([[1, 1], [2, 2], [3, 3], [4, 4], [5, 5]])
     assert ex.compute_pair_stats(five, five) == ex.PairsStats(5, 0, 0, 5, 5)
@@ -352,7 +358,16 @@ class MockBackend:
     def __init__(self):
         self.size, self.dim, self.log = 0, 0, []
 
-    def _result(self, epsilon):
+    def load_exponential(self, size, dim, lam=40.0, value_range=10.0):
+        self.size, self.dim = size, dim
+        self.log.append(("exp", size, dim, lam, value_range))
+
+    def load_file(self, path):
+        self.size, self.dim = 100000, 15
+        self.log.append(("file", str(path)))
+
+    def run(self, epsilon, save_pairs=False):
+        self.log.append(("run", epsilon, save_pairs))
         r = fp.Results()
         r.TFLOPS = 1.0
         r.pairsFound = r.pairsStored = int(epsilon * self.size) + self.size
@@ -360,19 +375,9 @@ class MockBackend:
         r.paddedProblemShape = fp.mmaShape(self.size, self.size, self.dim)
         return r
 
-    def runFromExponentialDataset(self, size, dim, e_lambda, e_range, epsilon, save_pairs):
-        self.size, self.dim = size, dim
-        self.log.append(("exp", size, dim, e_lambda, e_range, epsilon, save_pairs))
-        return self._result(epsilon)
-
-    def runFromFile(self, filename, epsilon, save_pairs):
-        self.size, self.dim = 100000, 15
-        self.log.append(("file", filename, epsilon, save_pairs))
-        return self._result(epsilon)
-
-    def reRun(self, epsilon, save_pairs):
-        self.log.append(("rerun", epsilon, save_pairs))
-        return self._result(epsilon)
+    def epsilon_for(self, target, sample_rows=None):
+        self.log.append(("search", target, sample_rows))
+        return float(target), float(target), 5
 
 
 def reference_record_keys():
@@ -382,15 +387,16 @@ def reference_record_keys():
     return set(rec), set(rec["results"]), gold
 
 
-def test_experiment_runner_writes_the_reference_result_schema(tmp_path):
+def test_sweep_driver_writes_the_reference_result_schema(tmp_path):
     from fasted_amd import experiments as ex
 
     top, inner, _ = reference_record_keys()
     backend = MockBackend()
-    runner = ex.ExperimentRunner(backend, output_dir=str(tmp_path))
+    driver = ex.SweepDriver(backend, output_dir=str(tmp_path))
 
-    # size x dimensionality sweep: 3 timed runs per shape, dataset built once per shape
-    path = runner.run_speed_sweeps_exponential_data_experiment(sizes=[1000, 2154], dims=[64, 128])
+    # size x dimensionality sweep: dataset built once per shape, 3 timed runs each
+    path = driver.exponential_sweep(sizes=[1000, 2154], dims=[64, 128])
+    assert re.fullmatch(r"ExpoDataSpeedVsSize_\d+\.json", os.path.basename(path))
     records = json.load(open(path))
     assert len(records) == 2 * 2 * 3
     for r in records:
@@ -400,42 +406,48 @@ def test_experiment_runner_writes_the_reference_result_schema(tmp_path):
     assert [r["iteration"] for r in records[:3]] == [0, 1, 2]
     builds = [e for e in backend.log if e[0] == "exp"]
     assert [(e[1], e[2]) for e in builds] == [(1000, 64), (1000, 128), (2154, 64), (2154, 128)]
-    assert all(e[3:5] == (40, 10) for e in builds)  # lambda 40, range 10 (experiments.py:556-557)
-    assert len([e for e in backend.log if e[0] == "rerun"]) == 8
-
-    # selectivity experiment: epsilon found per target (selectivity == epsilon for the mock), 3 runs each
+    assert all(e[3:5] == (40.0, 10.0) for e in builds)  # lambda 40, range 10 (experiments.py:556-557)
+    assert len([e for e in backend.log if e[0] == "run"]) == 12
+    # the default grid is the reference's: 10 log-spaced sizes x 7 dimensionalities
     backend.log.clear()
-    path = runner.run_selectivity_vs_speed_experiment([1, 10, 100], size=5000, dim=64)
+    driver.exponential_sweep(repetitions=0)
+    builds = [e for e in backend.log if e[0] == "exp"]
+    assert [e[1] for e in builds[::7]] == [1000, 2154, 4642, 10000, 21544, 46416, 100000, 215443, 464159, 1000000]
+    assert [e[2] for e in builds[:7]] == [64, 128, 256, 512, 1024, 2048, 4096]
+
+    # selectivity sweep: one build, one native search per target (epsilon == selectivity for the mock), 3 runs each
+    backend.log.clear()
+    path = driver.selectivity_sweep([1, 10, 100], size=5000, dim=64, sample_rows=512)
     records = json.load(open(path))
     assert len(records) == 9 and [r["selectivity"] for r in records[::3]] == [1, 10, 100]
-    for r in records:
-        assert ex.within_percent(r["epsilon"], r["selectivity"], 0.011)
-    assert len([e for e in backend.log if e[0] == "exp"]) == 1  # one build, everything else reRun
+    assert all(r["epsilon"] == r["selectivity"] for r in records)
+    assert [e for e in backend.log if e[0] in ("exp", "search")] == [
+        ("exp", 5000, 64, 40.0, 10.0), ("search", 1, 512), ("search", 10, 512), ("search", 100, 512)]
 
-    # known epsilons on a file: rebuilt for every run, pairs saved on the first run of a parameter set only
+    # known epsilons on a file: loaded once, pairs saved by the first run of a parameter set only
     backend.log.clear()
-    params = [ex.SearchParameters(64, 1.2, True), ex.SearchParameters(128, 3.4, False)]
-    path = runner.run_real_dataset_known_epsilons_experiments("base", "data.csv", params, num_repetitions=2)
+    path = driver.file_runs("base/data.csv", [(64, 1.2), (128, 3.4)], repetitions=2, save_pairs=True)
     assert os.path.basename(path).startswith("data.csv_results_")
-    assert [e[1:] for e in backend.log] == [(b"base/data.csv", 1.2, True), (b"base/data.csv", 1.2, False),
-                                            (b"base/data.csv", 3.4, False), (b"base/data.csv", 3.4, False)]
+    assert backend.log == [("file", "base/data.csv"), ("run", 1.2, True), ("run", 1.2, False), ("run", 3.4, True),
+                           ("run", 3.4, False)]
 
-    # epsilon finder over datasets: a dictionary of record lists keyed by dataset
-    path = runner.run_real_datasets_epsilon_finder_experiments([1, 10], base_path="base", datasets=["a.txt", "b.txt"])
+    # epsilon search over datasets: a dictionary of record lists keyed by dataset
+    path = driver.file_epsilon_search(["base/a.txt", "base/b.txt"], [1, 10])
     by_dataset = json.load(open(path))
     assert set(by_dataset) == {"a.txt", "b.txt"} and all(len(v) == 2 for v in by_dataset.values())
 
 
-def test_time_trials_skip_failed_runs():
+def test_timed_runs_skip_failed_runs():
     from fasted_amd import experiments as ex
 
-    calls = []
+    class Flaky(MockBackend):
+        def run(self, epsilon, save_pairs=False):
+            if len([e for e in self.log if e[0] == "run"]) == 1:
+                self.log.append(("run", epsilon, save_pairs))
+                raise RuntimeError("device lost")
+            return super().run(epsilon, save_pairs)
 
-    def finder(eps, save):
-        calls.append((eps, save))
-        if len(calls) == 2:
-            raise RuntimeError("device lost")
-        return fp.Results()
-
-    out = ex.ExperimentRunner(None).run_time_trials(finder, [ex.SearchParameters(1, 0.5, True)], 3)
-    assert [e.iteration for e in out] == [0, 2] and calls == [(0.5, True), (0.5, False), (0.5, False)]
+    backend = Flaky()
+    out = ex.SweepDriver(backend).timed_runs(1, 0.5, 3, save_pairs=True)
+    assert [r["iteration"] for r in out] == [0, 2]
+    assert [e[1:] for e in backend.log] == [(0.5, True), (0.5, False), (0.5, False)]

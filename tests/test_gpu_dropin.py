@@ -95,7 +95,7 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     """fasted_find_epsilon follows the reference's bound-then-bisect search probe for probe: the
     Python mirror driven by count-only probes lands on the same epsilon."""
     import fasted_amd
-    from fasted_amd import experiments as ex
+    from oracle import epsilon_search as ex
 
     n, d = 6000, 64
     assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
@@ -125,7 +125,7 @@ def test_sampled_epsilon_search(lib):
     import ctypes
 
     import fasted_amd
-    from fasted_amd import experiments as ex
+    from oracle import epsilon_search as ex
 
     n, d = 20000, 64
     assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
@@ -156,8 +156,8 @@ def test_experiment_sweep_reproduces_the_reference_result_records(lib, tmp_path)
         gold = json.load(f)["sweep"]
     sizes = sorted({r["results"]["inputProblemShape"]["m"] for r in gold})
     dims = sorted({r["results"]["inputProblemShape"]["k"] for r in gold})
-    runner = ex.ExperimentRunner(lib, output_dir=str(tmp_path))
-    records = json.load(open(runner.run_speed_sweeps_exponential_data_experiment(sizes=sizes, dims=dims, iterations=1)))
+    driver = ex.SweepDriver(ex.LibraryBackend(lib), output_dir=str(tmp_path))
+    records = json.load(open(driver.exponential_sweep(sizes=sizes, dims=dims, repetitions=1)))
     key = lambda r: (r["results"]["inputProblemShape"]["m"], r["results"]["inputProblemShape"]["k"])
     ours = {key(r): r for r in records}
     assert len(ours) == len(gold)
