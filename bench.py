@@ -257,8 +257,17 @@ def main():
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": traffic, "traffic_detail": traffic_detail},
     }
-    if not args.no_epilogue and st.pairsStored == st.pairsFound:
-        out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
+    # Parity is part of the measurement: a line whose pair set fails the check (a sampled pair outside the
+    # relative 1e-3 band around epsilon, a pair buffer that overflowed so that nothing could be checked, a
+    # symmetric-mode count that differs) says so and the process exits non-zero.
+    problems = []
+    if not args.no_epilogue:
+        if st.pairsStored == st.pairsFound:
+            out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
+            if out["config"]["parity_vs_fp64"]["outside_band"] > 0:
+                problems.append("sampled pairs outside the epsilon band")
+        else:
+            problems.append("pair buffer overflowed: parity not checked")
     if not args.no_epilogue and not args.no_symmetric_option:
         # Not part of `value`: the opt-in FASTED_SYMMETRIC mode computes only the tiles on and above the
         # diagonal (same pair set).  Its rate is 2*N^2*D over its time, i.e. an *effective* figure: the
@@ -270,9 +279,18 @@ def main():
             "ms_per_step": sym_ms, "effective_tflops": flops / (sym_ms / 1000.0) / 1e12,
             "pairs_found": int(sym.pairsFound), "same_pair_count": bool(sym.pairsFound == st.pairsFound),
             "note": "opt-in, not the headline: about half of 2*N^2*D is actually executed"}
+        if sym.pairsFound != st.pairsFound:
+            problems.append("symmetric mode found a different number of pairs")
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
+    if not args.no_epilogue:
+        out["config"]["parity_ok"] = not problems
+        if problems:
+            out["config"]["parity_problems"] = problems
     print(json.dumps(out))
+    if problems:
+        print("parity check failed: " + "; ".join(problems), file=sys.stderr)
+        sys.exit(3)
 
 
 if __name__ == "__main__":
