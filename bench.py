@@ -157,6 +157,68 @@ def cpu_baseline(torch, pts, eps, budget_s=15.0):
     }
 
 
+class ClockSampler:
+    """Shader clock and board power of GPU 0 while the timed steps run, read from the driver's sysfs files
+    (pp_dpm_sclk marks the current clock with '*', hwmon power1_input is microwatts, mem_busy_percent is
+    the driver's memory-controller activity) by a thread that makes
+    no GPU call.  The MFMA rate of a long join is set by the clock the power limit allows, not by 2.4 GHz."""
+
+    def __init__(self, interval=0.05):
+        import glob
+        import threading
+        self.interval = interval
+        dev = "/sys/class/drm/card0/device"
+        self.sclk = dev + "/pp_dpm_sclk"
+        power = glob.glob(dev + "/hwmon/hwmon*/power1_input") + glob.glob(dev + "/hwmon/hwmon*/power1_average")
+        cap = glob.glob(dev + "/hwmon/hwmon*/power1_cap")
+        self.power = power[0] if power else None
+        self.cap = cap[0] if cap else None
+        self.busy = dev + "/mem_busy_percent"
+        self.mhz, self.watts, self.mem = [], [], []
+        self._stop = threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _read_once(self):
+        try:
+            with open(self.sclk) as f:
+                for line in f:
+                    if "*" in line:
+                        self.mhz.append(float(line.split(":")[1].lower().split("mhz")[0]))
+            if self.power:
+                with open(self.power) as f:
+                    self.watts.append(float(f.read()) / 1e6)
+            with open(self.busy) as f:
+                self.mem.append(float(f.read()))
+        except (OSError, ValueError, IndexError):
+            pass
+
+    def _run(self):
+        while not self._stop.wait(self.interval):
+            self._read_once()
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def summary(self):
+        def stat(v):
+            return {"mean": sum(v) / len(v), "min": min(v), "max": max(v)} if v else None
+        cap = None
+        try:
+            if self.cap:
+                with open(self.cap) as f:
+                    cap = float(f.read()) / 1e6
+        except (OSError, ValueError):
+            pass
+        return {"sclk_mhz": stat(self.mhz), "power_w": stat(self.watts), "power_cap_w": cap,
+                "mem_busy_percent": stat(self.mem),
+                "samples": len(self.mhz), "interval_s": self.interval}
+
+
 def load_traffic(name):
     """Bytes below the L2 per join-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
     and scaled by a plain copy kernel (committed under profiles/); None when not measured."""
@@ -229,10 +291,11 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    stats = [step() for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    with ClockSampler() as clocks:
+        t0 = time.perf_counter()
+        stats = [step() for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
 
     ms_per_step = wall * 1000.0 / args.steps
     flops = 2.0 * n * n * d
@@ -252,7 +315,7 @@ def main():
                    "mean_neighbours": (st.pairsFound - n) / n, "pairs_per_s": st.pairsFound / (ms_per_step / 1000.0),
                    "pct_of_fp16_peak": 100.0 * tflops / PEAK_FP16_TFLOPS, "tiles": int(st.tiles),
                    "sum_squared_ms": sums_ms, "join_kernel_ms": join_ms, "epilogue": not args.no_epilogue,
-                   "accumulate": "f32", "peak_used_tflops": PEAK_FP16_TFLOPS},
+                   "accumulate": "f32", "peak_used_tflops": PEAK_FP16_TFLOPS, "clocks": clocks.summary()},
         "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": traffic, "traffic_detail": traffic_detail},

@@ -8,7 +8,7 @@ namespace fasted {
 
 constexpr int kTile = 256;       // points per tile side (queries x candidates)
 constexpr int kSlabK = 64;       // halves of K staged in LDS per pipeline stage
-constexpr int kRaster = 16;      // tiles per side of a raster square
+constexpr int kSquareTiles = 256; // tiles of a super-square of the work queues: one per workgroup of a full chip
 
 struct JoinLaunch {
     const void* queries;         // FP16 rows

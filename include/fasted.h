@@ -181,8 +181,8 @@ int fasted_sum_squared_device(const void* d_points, long long n, int d, long lon
  * (source/rasterizer/onDemandRasterizer.cuh:78-108). */
 int fasted_raster_coord(unsigned long long idx, long long n, int* row, int* col);
 unsigned long long fasted_raster_count(long long n);
-/* The same for a FASTED_SYMMETRIC join: only the 16x16-tile squares on and above the diagonal are
- * enumerated (row-major over the upper triangle), and tiles below the diagonal inside the diagonal squares
+/* The same for a FASTED_SYMMETRIC join: only the super-squares (32 x 8 tiles) that reach the diagonal or
+ * lie above it are enumerated (row by row), and tiles below the diagonal inside those squares
  * return 2 like padding tiles.  No counterpart in the reference, which always walks the full grid
  * (source/rasterizer/onDemandRasterizer.cuh:50-71). */
 int fasted_raster_coord_symmetric(unsigned long long idx, long long n, int* row, int* col);

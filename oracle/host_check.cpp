@@ -126,13 +126,14 @@ static void check_data_layer(const char* csvPath) {
 }
 
 static void check_tile_order() {
-    // every tile of the grid exactly once, for the 256x256 kernel's 4 x 8 sub-rectangles and for other cuts
+    // every tile of the grid exactly once, for the 256x256 kernel's 8 x 4 sub-rectangles and for other cuts
     const struct {
         long long nq, nc;
         int tm, tn, sr, sc;
         bool upper;
-    } cases[] = {{1, 1, 256, 256, 4, 8, false},      {4097, 4097, 256, 256, 4, 8, false}, {9000, 3000, 256, 256, 4, 8, false},
-                 {10000, 10000, 256, 256, 4, 8, true}, {5000, 7000, 256, 128, 4, 16, false}, {6000, 6000, 128, 128, 8, 16, false}};
+    } cases[] = {{1, 1, 256, 256, 8, 4, false},       {4097, 4097, 256, 256, 8, 4, false}, {9000, 3000, 256, 256, 8, 4, false},
+                 {10000, 10000, 256, 256, 8, 4, true}, {70000, 70000, 256, 256, 8, 4, true}, {10000, 10000, 256, 256, 4, 8, true},
+                 {5000, 7000, 256, 128, 4, 16, false}, {6000, 6000, 128, 128, 8, 16, false}, {20000, 20000, 256, 256, 16, 2, true}};
     for (const auto& c : cases) {
         const fasted::TileOrder o = fasted::make_tile_order(c.nq, c.nc, c.tm, c.tn, c.sr, c.sc, c.upper);
         std::set<std::pair<unsigned, unsigned>> seen;
@@ -145,6 +146,7 @@ static void check_tile_order() {
                 CHECK(seen.insert({tr, tc}).second);
                 ++real;
             }
+        CHECK((o.upperOnly != 0) == c.upper);
         if (!o.upperOnly) {
             CHECK(real == (unsigned long long)o.tileRows * o.tileCols);
         } else {

@@ -194,29 +194,43 @@ def test_symmetric_tile_queues_cover_the_upper_triangle_exactly_once(lib, n):
             seen[row.value // 256, col.value // 256] += 1
     assert lib.fasted_raster_coord_symmetric(total, n, ctypes.byref(row), ctypes.byref(col)) == 0
     assert np.array_equal(seen, np.triu(np.ones((tiles, tiles), dtype=np.int32)))
-    squares = -(-tiles // 16)
-    assert total == 256 * squares * (squares + 1) // 2 <= lib.fasted_raster_count(n)
+    if tiles >= 64:
+        # super-squares are 32 x 8 tiles: row i of them keeps the squares from column 4 * i on
+        square_rows, square_cols = -(-tiles // 32), -(-tiles // 8)
+        expected = 256 * sum(square_cols - 4 * i for i in range(square_rows))
+    else:
+        # small matrices: 16 x 16 super-squares, the upper triangle of them
+        squares = -(-tiles // 16)
+        expected = 256 * squares * (squares + 1) // 2
+    assert total == expected <= lib.fasted_raster_count(n)
 
 
 def test_tile_queue_locality(lib):
-    """32 consecutive positions of one queue are one 4 x 8 block of tiles (one XCD's share of a
-    16 x 16 super-square), and the 8 queues together tile that super-square."""
-    n = 256 * 48
+    """32 consecutive positions of one queue are one block of tiles (one XCD's share of a super-square), the 8
+    queues together tile that super-square, and consecutive super-squares follow each other along the
+    candidates (the query panels stay).  Matrices of 64 x 64 tiles and more: blocks of 8 x 4, super-squares of
+    32 x 8; smaller ones: 4 x 8 and 16 x 16."""
     row, col = ctypes.c_int(), ctypes.c_int()
-    for square in (0, 1, 4):
-        cover = set()
-        for q in range(8):
-            block = []
-            for t in range(32):
-                idx = (square * 32 + t) * 8 + q
-                assert lib.fasted_raster_coord(idx, n, ctypes.byref(row), ctypes.byref(col)) == 1
-                block.append((row.value // 256, col.value // 256))
-            r0, c0 = block[0]
-            assert block == [(r0 + t // 8, c0 + t % 8) for t in range(32)]
-            cover |= set(block)
-        rs, cs = min(r for r, _ in cover), min(c for _, c in cover)
-        assert cover == {(rs + i, cs + j) for i in range(16) for j in range(16)}
-        assert rs % 16 == 0 and cs % 16 == 0
+    for n_tiles, (br, bc), expected in ((96, (8, 4), [(0, 0), (0, 8), (0, 32), (32, 0), (32, 8)]),
+                                       (48, (4, 8), [(0, 0), (0, 16), (16, 16), (32, 0), (32, 16)])):
+        n = 256 * n_tiles
+        origins = []
+        squares = (0, 1, 4, 12, 13) if n_tiles == 96 else (0, 1, 4, 6, 7)
+        for square in squares:
+            cover = set()
+            for q in range(8):
+                block = []
+                for t in range(32):
+                    idx = (square * 32 + t) * 8 + q
+                    assert lib.fasted_raster_coord(idx, n, ctypes.byref(row), ctypes.byref(col)) == 1
+                    block.append((row.value // 256, col.value // 256))
+                r0, c0 = block[0]
+                assert block == [(r0 + t // bc, c0 + t % bc) for t in range(32)]
+                cover |= set(block)
+            rs, cs = min(r for r, _ in cover), min(c for _, c in cover)
+            assert cover == {(rs + i, cs + j) for i in range(4 * br) for j in range(2 * bc)}
+            origins.append((rs, cs))
+        assert origins == expected
 
 
 # ---------------------------------------------------------------- LDS swizzle (host mirror)
