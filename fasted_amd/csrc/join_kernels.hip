@@ -50,6 +50,34 @@ static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
 // the 1M x 4096 workload than one transfer pinned in front of every 4 MFMAs)
 constexpr bool kSpread = false;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
+
+// Measurement builds (`make ablation`): the join kernel with parts compiled out, to see what each part
+// costs in time and in power.  Such a build computes wrong results; the library proper is built with 0.
+//   FASTED_ABLATE bit 0: the accumulators are not initialised
+//                 bit 1: no global -> LDS transfers once both LDS stages hold the first two slabs of the
+//                        workgroup's first tile (the matrix cores keep seeing real operand values)
+//                 bit 2: no LDS fragment reads (the operand registers hold whatever they held)
+//   FASTED_ABLATE_PANELS k > 0: every tile reads the panels (row % k, col % k): the whole join touches
+//                        k panels of 256 points only, so they stay in the Infinity Cache (or the L2)
+#ifndef FASTED_ABLATE
+#define FASTED_ABLATE 0
+#endif
+#ifndef FASTED_ABLATE_PANELS
+#define FASTED_ABLATE_PANELS 0
+#endif
+constexpr bool kNoInit = (FASTED_ABLATE & 1) != 0, kNoTransfers = (FASTED_ABLATE & 2) != 0,
+               kNoFragments = (FASTED_ABLATE & 4) != 0;
+__device__ __forceinline__ unsigned panel_of(unsigned tile) {
+    return FASTED_ABLATE_PANELS > 0 ? tile % (unsigned)(FASTED_ABLATE_PANELS > 0 ? FASTED_ABLATE_PANELS : 1) : tile;
+}
+__device__ __forceinline__ half8 fragment(const unsigned char* p) {
+    if (kNoFragments) {
+        half8 v;
+        asm volatile("" : "=v"(v) : "v"((unsigned)(size_t)p));
+        return v;
+    }
+    return *reinterpret_cast<const half8*>(p);
+}
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
 // Operand rows of the 256x256 kernel are 128 bytes (a 64-wide k-slab): see lds_swizzle128 in
@@ -309,8 +337,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // One 1-KiB global->LDS transfer of this wave (global_load_lds_dwordx4: no registers in between);
     // j = 0..7 alternates query / candidate rows.  Lane l lands in row l/8, chunk slot l%8 of the
     // 8 rows the instruction fills; wave w owns rows [32w, 32w+32) of both operands.
+    bool filling = true;  // (measurement builds only)
     auto issue_load = [&](const char* slabA, const char* slabB, const unsigned (&oA)[4], const unsigned (&oB)[4],
                           int stage, int j) {
+        if (kNoTransfers && !filling) return;
         const int i = j >> 1;
         const unsigned dst = ldsBase + (unsigned)(stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes);
         // Written as instructions: the slab's address in scalar registers, the lane's offset a 32-bit vector
@@ -351,10 +381,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     unsigned offA[4], offB[4];
     tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB, true);
-    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)tr * kTile * p.ldQ16);
-    const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)tc * kTile * p.ldC16);
+    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(tr) * kTile * p.ldQ16);
+    const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(tc) * kTile * p.ldC16);
 #pragma unroll
     for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0, j);
+    if (kNoTransfers) {
+        const int second = p.nSlabs > 1 ? kRowBytes : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) issue_load(gA + second, gB + second, offA, offB, 1, j);
+        filling = false;
+    }
     issue_sums((int)tr * kTile, (int)tc * kTile, 0);
     unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
     if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
@@ -390,7 +426,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             for (int fi = 0; fi < kFragRows; ++fi) {
                 const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16);
 #pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) acc[fi][fj] = hq + hc[fj];  // commutative: the same for (q, c) and (c, q)
+                for (int fj = 0; fj < kFragCols; ++fj) {
+                    if (kNoInit)
+                        asm volatile("" : "=v"(acc[fi][fj]));
+                    else
+                        acc[fi][fj] = hq + hc[fj];  // commutative: the same for (q, c) and (c, q)
+                }
             }
         }
 
@@ -409,15 +450,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
-                b[0][fj] = *reinterpret_cast<const half8*>(buf + bOff[0] + fj * 16 * kRowBytes);
+                b[0][fj] = fragment(buf + bOff[0] + fj * 16 * kRowBytes);
 #pragma unroll
             for (int fi = 0; fi < 4; ++fi)
-                aLo[fi] = *reinterpret_cast<const half8*>(buf + aOff[0] + fi * 16 * kRowBytes);
+                aLo[fi] = fragment(buf + aOff[0] + fi * 16 * kRowBytes);
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi)
-                    aHi[fi] = *reinterpret_cast<const half8*>(buf + aOff[ks] + (fi + 4) * 16 * kRowBytes);
+                    aHi[fi] = fragment(buf + aOff[ks] + (fi + 4) * 16 * kRowBytes);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi) {
@@ -433,10 +474,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 if (ks == 0) {
 #pragma unroll
                     for (int fj = 0; fj < kFragCols; ++fj)
-                        b[1][fj] = *reinterpret_cast<const half8*>(buf + bOff[1] + fj * 16 * kRowBytes);
+                        b[1][fj] = fragment(buf + bOff[1] + fj * 16 * kRowBytes);
 #pragma unroll
                     for (int fi = 0; fi < 4; ++fi)
-                        aLo[fi] = *reinterpret_cast<const half8*>(buf + aOff[1] + fi * 16 * kRowBytes);
+                        aLo[fi] = fragment(buf + aOff[1] + fi * 16 * kRowBytes);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -469,8 +510,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const bool more = ntr != kNoTile;
         if (more) {
             tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB, false);
-            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)ntr * kTile * p.ldQ16);
-            gB = reinterpret_cast<const char*>(p.ptsC + (long long)ntc * kTile * p.ldC16);
+            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(ntr) * kTile * p.ldQ16);
+            gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(ntc) * kTile * p.ldC16);
             issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
         }
         slab_step(stage, more, gA, gB, offA, offB);

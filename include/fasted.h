@@ -130,8 +130,9 @@ int fasted_self_join_device(const void* d_points, long long n, int d, long long 
 
 /* fasted_self_join_device for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The queue
- * heads, the pair counter and the squared norms live in a device array that is part of the library image
- * (4 KiB + 16 MiB per GPU, held until the process ends) instead of allocated workspace; the call makes no
+ * heads, the pair counter, the squared norms and the per-point accumulator start values live in a device
+ * array that is part of the library image (4 KiB + 32 MiB per GPU, held until the process ends) instead of
+ * allocated workspace; the call makes no
  * hipMalloc / hipFree and calls no allocating library routine.  Limits, each refused with an error:
  * n <= 4 194 304 points; FASTED_SORT_PAIRS (the sort needs device buffers; the pairs come back in
  * arbitrary order) and FASTED_SKIP_SUMS are not accepted.  Every call on one GPU shares that GPU's array:
