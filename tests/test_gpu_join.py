@@ -396,3 +396,42 @@ def test_join_is_deterministic_over_many_tiles_per_workgroup(fasted):
     diff = truth != mask
     rel = (d2[diff].sqrt() - eps).abs() / eps
     assert int((rel > 1e-3).sum()) == 0, (int(diff.sum()), float(rel.max()))
+
+
+def test_tall_tile_order_exact_pair_sets(fasted):
+    """From 64 x 64 tiles on, the work queues walk super-squares of 32 x 8 tiles.  Integer coordinates make the
+    join exact, so on a ragged matrix of 65 x 65 tiles the default order, the symmetric option (upper part of
+    the tall super-squares, mirrored) and a rectangular two-set join (65 x 3 tiles: most super-square positions
+    are padding) must each give exactly the pair list of a blockwise FP64 computation."""
+    import torch
+    from fasted_amd import find_pairs as fp
+
+    n, d, nc = 64 * 256 + 37, 64, 600
+    bits = datasets.small_integers(n, d, high=3, seed=91)
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    x = pts.view(torch.float16).double()
+    norms = (x * x).sum(1)
+    d2_head = norms[:64, None] + norms[None, :64] - 2.0 * x[:64] @ x[:64].T
+    target = torch.sort(d2_head[torch.triu_indices(64, 64, 1).unbind()]).values[30]
+    eps = float(torch.sqrt(target + 0.5))
+
+    def truth(cols):
+        out = []
+        for r0 in range(0, n, 4096):
+            blk = norms[r0:r0 + 4096, None] + norms[None, :cols] - 2.0 * x[r0:r0 + 4096] @ x[:cols].T
+            q, c = torch.nonzero(blk <= eps * eps, as_tuple=True)
+            out.append(torch.stack([q + r0, c], 1))
+        return torch.cat(out).to(torch.int32)
+
+    want = truth(n)
+    cap = int(want.shape[0]) + 1024
+    for flags in (fp.FASTED_SORT_PAIRS, fp.FASTED_SORT_PAIRS | fp.FASTED_SYMMETRIC):
+        pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+        st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, flags=flags)
+        assert st.pairsFound == st.pairsStored == want.shape[0]
+        assert bool((pairs[: st.pairsStored] == want).all())
+    want2 = truth(nc)
+    pairs = torch.empty((int(want2.shape[0]) + 1024, 2), dtype=torch.int32, device="cuda")
+    st = fasted.join_device(pts.data_ptr(), n, d, pts.data_ptr(), nc, d, d, eps, pairs.data_ptr(), pairs.shape[0])
+    assert st.pairsFound == st.pairsStored == want2.shape[0]
+    assert bool((pairs[: st.pairsStored] == want2).all())
