@@ -607,9 +607,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 // Extraction, one word of hit bits after the other.  Each round takes the first remaining hit
                 // of every lane that has one: the lanes form a mask in scalar registers, a lane's record goes
                 // behind those of the lanes before it, the wave's fill count moves on by the number of lanes.
-#pragma unroll 1
+#pragma unroll
                 for (int fp = 0; fp < kFragRows / 2; ++fp) {
-                    unsigned w = fp == 0 ? hits[0] : fp == 1 ? hits[1] : fp == 2 ? hits[2] : hits[3];
+                    unsigned w = hits[fp];
                     for (;;) {
                         const unsigned long long lanes = __builtin_amdgcn_ballot_w64(w != 0u);
                         if (lanes == 0ull) break;
