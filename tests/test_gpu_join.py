@@ -120,7 +120,7 @@ def test_plumbing_config_full_fp64_check(fasted):
     check_against_fp64(bits, n, eps, model)
 
 
-@pytest.mark.parametrize("n,d", [(1, 64), (2, 64), (255, 64), (257, 128), (1000, 320), (5000, 64)])
+@pytest.mark.parametrize("n,d", [(1, 64), (2, 64), (255, 64), (257, 128), (1000, 320), (5000, 64), (300, 16384), (513, 8000)])
 def test_ragged_sizes(fasted, n, d):
     bits = datasets.uniform_bytes(n, d, seed=n)
     eps = datasets.epsilon_for_neighbours(bits, min(8, max(n - 1, 0) / 2)) if n > 2 else 0.5
