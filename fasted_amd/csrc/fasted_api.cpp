@@ -253,7 +253,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     float sortMs = 0.f;
     if ((flags & FASTED_SORT_PAIRS) && cnt[1] > 1) {
         const auto w0 = std::chrono::steady_clock::now();
-        const hipError_t e = fasted::sort_pairs_row_major(dPairs, cnt[1], stream, &g_sortWs);
+        const hipError_t e = fasted::sort_pairs_row_major(dPairs, cnt[1], stream, &g_sortWs, q.n, c.n);
         if (e != hipSuccess) {
             (void)hipGetLastError();
             if (!sortMayFail) hip_check(e, "row-major sort of the pairs");
@@ -433,7 +433,7 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
             before = after;
         }
         const unsigned long long kept = std::min(before, devCap);
-        if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute, &g_sortWs));
+        if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute, &g_sortWs, n, n));
         HIP_CHECK(hipStreamSynchronize(dev.compute));
         const unsigned long long take = std::min(kept, cap - storedAll);
         if (take)

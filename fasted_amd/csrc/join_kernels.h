@@ -68,8 +68,10 @@ struct SortBuffers {
 };
 // Row-major sort of `count` stored pairs (pair_sort.hip); synchronises the stream.  With ws == nullptr the
 // buffers are allocated and freed inside the call.  On failure (no memory for the buffers) the pairs are left
-// as they were, unsorted.
-hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws = nullptr);
+// as they were, unsorted.  nQueries / nCandidates bound the indices (0: unknown): the sort then only runs over
+// the bits the indices can occupy.
+hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws = nullptr,
+                                long long nQueries = 0, long long nCandidates = 0);
 // Device bytes a sort of `count` pairs needs beside the pairs themselves.
 size_t sort_scratch_bytes(unsigned long long count);
 

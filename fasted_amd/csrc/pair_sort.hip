@@ -3,8 +3,9 @@
 //
 // The reference sorts its pair buffer with thrust::sort and Pair::operator< (query index,
 // then candidate index; source/pair.cuh:39-45,151-158).  A pair is 8 bytes with the query
-// index in the low word, so rotating each record by 32 bits turns that order into plain
-// unsigned 64-bit order: rotate, radix sort, rotate back.
+// index in the low word; packed as (query << bits of a candidate index) | candidate that order is plain
+// unsigned order on the low bits of a 64-bit key: pack, radix sort over just those bits (42 instead of 64
+// for two million points: 6 passes of 8 bits instead of 8), unpack.
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -14,13 +15,29 @@
 namespace fasted {
 namespace {
 
-__global__ void rotate_pairs_kernel(const unsigned long long* __restrict__ in, unsigned long long* __restrict__ out,
-                                    unsigned long long count) {
+// record (candidate << 32 | query) -> key (query << candidateBits | candidate), and back
+__global__ void pack_pairs_kernel(const unsigned long long* __restrict__ in, unsigned long long* __restrict__ out,
+                                  unsigned long long count, int candidateBits) {
     const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
     for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
         const unsigned long long v = in[i];
-        out[i] = (v << 32) | (v >> 32);
+        out[i] = ((v & 0xffffffffull) << candidateBits) | (v >> 32);
     }
+}
+__global__ void unpack_pairs_kernel(const unsigned long long* __restrict__ in, unsigned long long* __restrict__ out,
+                                    unsigned long long count, int candidateBits) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        const unsigned long long k = in[i];
+        out[i] = ((k & ((1ull << candidateBits) - 1ull)) << 32) | (k >> candidateBits);
+    }
+}
+
+int index_bits(long long n) {  // bits of the largest index of n items; 32 when n is not known
+    if (n <= 0 || n > (1ll << 32)) return 32;
+    int b = 1;
+    while ((1ll << b) < n) ++b;
+    return b;
 }
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -107,7 +124,8 @@ size_t sort_scratch_bytes(unsigned long long count) {
     return needTemp + (size_t)count * sizeof(unsigned long long);
 }
 
-hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws) {
+hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream_t stream, SortBuffers* ws,
+                                long long nQueries, long long nCandidates) {
     if (count < 2) return hipSuccess;
     SortBuffers local;
     SortBuffers* const b = ws ? ws : &local;
@@ -115,15 +133,17 @@ hipError_t sort_pairs_row_major(void* pairs, unsigned long long count, hipStream
     auto* keys = static_cast<unsigned long long*>(pairs);
     auto* alt = static_cast<unsigned long long*>(b->alt);
     if (e == hipSuccess) {
+        const int candidateBits = index_bits(nCandidates);
+        const unsigned keyBits = (unsigned)(candidateBits + index_bits(nQueries));
         size_t tempBytes = b->tempBytes;
-        rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count);
-        e = rocprim::radix_sort_keys(b->temp, tempBytes, keys, alt, (size_t)count, 0u, 64u, stream);
+        pack_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count, candidateBits);
+        e = rocprim::radix_sort_keys(b->temp, tempBytes, keys, alt, (size_t)count, 0u, keyBits, stream);
         if (e == hipSuccess) {
-            rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(alt, keys, count);
+            unpack_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(alt, keys, count, candidateBits);
             e = hipGetLastError();
         } else {
-            // the keys are still in place, rotated: put them back as they were
-            rotate_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count);
+            // the keys are still in place, packed: put the records back as they were
+            unpack_pairs_kernel<<<grid_for(count), 256, 0, stream>>>(keys, keys, count, candidateBits);
         }
     }
     const hipError_t s = hipStreamSynchronize(stream);
