@@ -46,9 +46,6 @@ constexpr int kLdsStage = kLdsNext + 16;            // staged pairs: one private
 constexpr int kWaveStagePairs = 384;                // 3 KiB of 8-byte records per wave
 constexpr int kLdsBytes = kLdsStage + 8 * kWaveStagePairs * 8;
 static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
-// false: the four transfers of half a k-step are issued in a cluster at its start (measured 1-3 % faster on
-// the 1M x 4096 workload than one transfer pinned in front of every 4 MFMAs)
-constexpr bool kSpread = false;
 constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
 
 // Measurement builds (`make ablation`): the join kernel with parts compiled out, to see what each part
@@ -227,6 +224,16 @@ __device__ __forceinline__ void transfers_landed_barrier() {
     __syncthreads();
 }
 
+// f(integral_constant<int, kBegin>) ... f(integral_constant<int, kEnd - 1>): a loop whose index is a constant
+// expression inside the body (an immediate operand of hand-written instructions needs one)
+template <int kBegin, int kEnd, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (kBegin < kEnd) {
+        f(std::integral_constant<int, kBegin>{});
+        static_for<kBegin + 1, kEnd>(f);
+    }
+}
+
 template <bool kEpilogue, bool kTall>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __shared__ __align__(16) unsigned char lds[kLdsBytes];
@@ -336,22 +343,29 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     // One 1-KiB global->LDS transfer of this wave (global_load_lds_dwordx4: no registers in between);
     // j = 0..7 alternates query / candidate rows.  Lane l lands in row l/8, chunk slot l%8 of the
-    // 8 rows the instruction fills; wave w owns rows [32w, 32w+32) of both operands.
+    // 8 rows the instruction fills.
     bool filling = true;  // (measurement builds only)
-    auto issue_load = [&](const char* slabA, const char* slabB, const unsigned (&oA)[4], const unsigned (&oB)[4],
-                          int stage, int j) {
+    // LDS byte address of this wave's first row in stage 0: wave w owns rows [32w, 32w+32) of both operands
+    const unsigned waveRows = ldsBase + (unsigned)(wave * 32 * kRowBytes);
+    auto issue_load = [&](auto jc, const char* slabA, const char* slabB, const unsigned (&oA)[4], const unsigned (&oB)[4],
+                          int stage) {
         if (kNoTransfers && !filling) return;
-        const int i = j >> 1;
-        const unsigned dst = ldsBase + (unsigned)(stage * kStageBytes + (j & 1) * kOperandBytes + (wave * 32 + i * 8) * kRowBytes);
-        // Written as instructions: the slab's address in scalar registers, the lane's offset a 32-bit vector
-        // register that never changes -- no vector arithmetic per transfer (left to the compiler, the
-        // addresses become loop-carried 64-bit vector pointers).  M0 holds the LDS destination.
+        constexpr int j = decltype(jc)::value;
+        constexpr int i = j >> 1;
+        constexpr unsigned within = (unsigned)((j & 1) * kOperandBytes + i * 8 * kRowBytes);
+        const unsigned stageRows = waveRows + (unsigned)(stage * kStageBytes);
+        // Written as instructions: M0 (the LDS destination) is formed by one scalar add with an immediate, the
+        // slab's address sits in scalar registers, the lane's offset is a 32-bit vector register that never
+        // changes -- no vector arithmetic per transfer (left to the compiler, the addresses become
+        // loop-carried 64-bit vector pointers, and M0 costs a scalar instruction or two more).
         if (j & 1)
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(oB[i]), "s"(slabB)
-                         : "memory", "m0");
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(stageRows), "n"(within),
+                         "v"(oB[i]), "s"(slabB)
+                         : "memory", "m0", "scc");
         else
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(oA[i]), "s"(slabA)
-                         : "memory", "m0");
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(stageRows), "n"(within),
+                         "v"(oA[i]), "s"(slabA)
+                         : "memory", "m0", "scc");
     };
 
     // Per-point halves (eps^2/4 - s/2) of a tile's 256 queries (waves 0-3) and 256 candidates (waves 4-7),
@@ -383,12 +397,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB, true);
     const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(tr) * kTile * p.ldQ16);
     const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(tc) * kTile * p.ldC16);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) issue_load(gA, gB, offA, offB, 0, j);
+    static_for<0, 8>([&](auto jc) { issue_load(jc, gA, gB, offA, offB, 0); });
     if (kNoTransfers) {
         const int second = p.nSlabs > 1 ? kRowBytes : 0;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) issue_load(gA + second, gB + second, offA, offB, 1, j);
+        static_for<0, 8>([&](auto jc) { issue_load(jc, gA + second, gB + second, offA, offB, 1); });
         filling = false;
     }
     issue_sums((int)tr * kTile, (int)tc * kTile, 0);
@@ -442,7 +454,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // scheduling barriers: the LDS reads for the next half are issued ahead of the MFMAs of
         // the current half, and the 8 global->LDS transfers of the following slab are issued during
         // the first k-step, four at the start of each of its halves: early, so that an L2 miss has the
-        // whole second k-step to land before the slab's barrier.
+        // whole second k-step to land before the slab's barrier (one transfer pinned in front of every 4 MFMAs
+        // instead measured 1-3 % slower on the 1M x 4096 workload).
         auto slab_step = [&](int stg, bool prefetch, const char* pA, const char* pB, const unsigned (&oA)[4],
                              const unsigned (&oB)[4]) {
             const unsigned char* const buf = lds + stg * kStageBytes;
@@ -460,15 +473,14 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 for (int fi = 0; fi < 4; ++fi)
                     aHi[fi] = fragment(buf + aOff[ks] + (fi + 4) * 16 * kRowBytes);
                 __builtin_amdgcn_sched_barrier(0);
+                if (ks == 0 && prefetch) static_for<0, 4>([&](auto jc) { issue_load(jc, pA, pB, oA, oB, stg ^ 1); });
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi) {
-                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, stg ^ 1, fi);
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
                     }
-                    if (ks == 0 && kSpread) __builtin_amdgcn_sched_barrier(0);  // keeps each transfer in front of its 4 MFMAs
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -480,16 +492,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         aLo[fi] = fragment(buf + aOff[1] + fi * 16 * kRowBytes);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                if (ks == 0 && prefetch) static_for<4, 8>([&](auto jc) { issue_load(jc, pA, pB, oA, oB, stg ^ 1); });
 #pragma unroll
                 for (int fi = 0; fi < 4; ++fi) {
-                    if (ks == 0 && prefetch) issue_load(pA, pB, oA, oB, stg ^ 1, 4 + fi);
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;
                         acc[fi + 4][fj] =
                             __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
                     }
-                    if (ks == 0 && kSpread) __builtin_amdgcn_sched_barrier(0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
