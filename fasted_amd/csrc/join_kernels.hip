@@ -422,30 +422,32 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         }
 
-        // the accumulators start at h_q + h_c, h = eps^2/4 - s/2 per point (see the epilogue): the tile's
-        // 512 values landed together with slab 0
+        // The accumulators start at h_q + h_c, h = eps^2/4 - s/2 per point (see the epilogue): the tile's
+        // 512 values landed together with slab 0.  Only the first row of blocks is set here; the others are
+        // set between the MFMAs of the tile's first k-step, one row of blocks ahead of the MFMAs that need it
+        // (a wave's vector instructions between its own MFMAs cost far less than on their own).
         floatx4 acc[kFragRows][kFragCols];
+        float hc[kFragCols];
+        const float* sQw;
         {
             const int ln = lane_now();
-            const float* const sQw =
-                reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + wr * kWaveRows + (ln >> 4) * 4;
+            sQw = reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + wr * kWaveRows + (ln >> 4) * 4;
             const float* const sCw =
                 reinterpret_cast<const float*>(lds + kLdsSums + sumsBuf * kSumsBytes) + kTile + wc * kWaveCols + (ln & 15);
-            float hc[kFragCols];
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj) hc[fj] = sCw[fj * 16];
-#pragma unroll
-            for (int fi = 0; fi < kFragRows; ++fi) {
-                const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16);
-#pragma unroll
-                for (int fj = 0; fj < kFragCols; ++fj) {
-                    if (kNoInit)
-                        asm volatile("" : "=v"(acc[fi][fj]));
-                    else
-                        acc[fi][fj] = hq + hc[fj];  // commutative: the same for (q, c) and (c, q)
-                }
-            }
         }
+        auto init_row = [&](int fi) {
+            const floatx4 hq = *reinterpret_cast<const floatx4*>(sQw + fi * 16);
+#pragma unroll
+            for (int fj = 0; fj < kFragCols; ++fj) {
+                if (kNoInit)
+                    asm volatile("" : "=v"(acc[fi][fj]));
+                else
+                    acc[fi][fj] = hq + hc[fj];  // commutative: the same for (q, c) and (c, q)
+            }
+        };
+        init_row(0);
 
         // One slab = 2 k-steps of 32; a k-step is two halves of 16 MFMAs (query blocks 0-3, then
         // 4-7, each against the 4 candidate blocks, query fragment held for 4 MFMAs, candidate blocks
@@ -456,8 +458,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // the first k-step, four at the start of each of its halves: early, so that an L2 miss has the
         // whole second k-step to land before the slab's barrier (one transfer pinned in front of every 4 MFMAs
         // instead measured 1-3 % slower on the 1M x 4096 workload).
-        auto slab_step = [&](int stg, bool prefetch, const char* pA, const char* pB, const unsigned (&oA)[4],
-                             const unsigned (&oB)[4]) {
+        auto slab_step = [&](auto firstc, int stg, bool prefetch, const char* pA, const char* pB,
+                             const unsigned (&oA)[4], const unsigned (&oB)[4]) {
+            constexpr bool first = decltype(firstc)::value;  // the tile's first slab also sets the accumulators
             const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[4], aHi[4], b[2][kFragCols];
 
@@ -481,6 +484,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
                     }
+                    if (first && ks == 0) init_row(fi + 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -501,13 +505,21 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         acc[fi + 4][fj] =
                             __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
                     }
+                    if (first && ks == 0 && fi < 3) init_row(fi + 5);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
 
-        for (int s = 0; s + 1 < p.nSlabs; ++s) {
-            slab_step(stage, true, gA + (s + 1) * kRowBytes, gB + (s + 1) * kRowBytes, offA, offB);
+        constexpr std::integral_constant<bool, true> kFirstSlab{};
+        constexpr std::integral_constant<bool, false> kLaterSlab{};
+        if (p.nSlabs > 1) {
+            slab_step(kFirstSlab, stage, true, gA + kRowBytes, gB + kRowBytes, offA, offB);
+            stage ^= 1;
+            transfers_landed_barrier();
+        }
+        for (int s = 1; s + 1 < p.nSlabs; ++s) {
+            slab_step(kLaterSlab, stage, true, gA + (s + 1) * kRowBytes, gB + (s + 1) * kRowBytes, offA, offB);
             stage ^= 1;
             transfers_landed_barrier();
         }
@@ -525,7 +537,11 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(ntc) * kTile * p.ldC16);
             issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
         }
-        slab_step(stage, more, gA, gB, offA, offB);
+        if (p.nSlabs == 1) {  // a single slab: all rows are set before it
+#pragma unroll
+            for (int fi = 1; fi < kFragRows; ++fi) init_row(fi);
+        }
+        slab_step(kLaterSlab, stage, more, gA, gB, offA, offB);
         stage ^= 1;
 
         if (kEpilogue) {
