@@ -75,6 +75,10 @@ __device__ __forceinline__ half8 fragment(const unsigned char* p) {
     }
     return *reinterpret_cast<const half8*>(p);
 }
+#ifndef FASTED_ROW_MAJOR_FIRST_SLAB
+#define FASTED_ROW_MAJOR_FIRST_SLAB 1
+#endif
+constexpr bool kRowMajorFirstSlab = FASTED_ROW_MAJOR_FIRST_SLAB != 0;
 constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
 
 // Operand rows of the 256x256 kernel are 128 bytes (a 64-wide k-slab): see lds_swizzle128 in
@@ -464,6 +468,66 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[4], aHi[4], b[2][kFragCols];
 
+            if constexpr (first && kRowMajorFirstSlab) {
+                // The tile's first slab goes through the rows of blocks one after the other, both k-steps of a
+                // row together (an element still receives k-step 0 before k-step 1): the 16 start values of row
+                // fi + 1 are formed between the 8 MFMAs of row fi, two vector instructions behind every MFMA,
+                // which is about what a wave issues for free there.  The rows' h_q are read ahead of the slab
+                // (into registers of accumulators that are not live yet).
+                floatx4 hq[kFragRows];
+                half8 a[2][2];
+                // what the first MFMAs need is read first (LDS reads complete in order)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    a[0][ks] = fragment(buf + aOff[ks]);
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj) b[ks][fj] = fragment(buf + bOff[ks] + fj * 16 * kRowBytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int fi = 1; fi < kFragRows; ++fi) hq[fi] = *reinterpret_cast<const floatx4*>(sQw + fi * 16);
+                static_for<0, kFragRows>([&](auto fic) {
+                    constexpr int fi = decltype(fic)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (fi < 4) {
+                        if (prefetch) {
+                            issue_load(std::integral_constant<int, 2 * fi>{}, pA, pB, oA, oB, stg ^ 1);
+                            issue_load(std::integral_constant<int, 2 * fi + 1>{}, pA, pB, oA, oB, stg ^ 1);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (fi + 1 < kFragRows) {
+                        a[(fi + 1) & 1][0] = fragment(buf + aOff[0] + (fi + 1) * 16 * kRowBytes);
+                        a[(fi + 1) & 1][1] = fragment(buf + aOff[1] + (fi + 1) * 16 * kRowBytes);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int fs = 0; fs < kFragCols; ++fs) {
+                            const int fj = ((fi + ks) & 1) ? kFragCols - 1 - fs : fs;
+                            acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[fi & 1][ks], b[ks][fj], acc[fi][fj], 0, 0, 0);
+                        }
+                    if constexpr (fi + 1 < kFragRows) {
+#pragma unroll
+                        for (int fj = 0; fj < kFragCols; ++fj) {
+                            if (kNoInit)
+                                asm volatile("" : "=v"(acc[fi + 1][fj]));
+                            else
+                                acc[fi + 1][fj] = hq[fi + 1] + hc[fj];
+                        }
+                        // the order asked of the scheduler: the two fragment reads, then MFMA, 2 adds, MFMA, 2 adds ...
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+                        for (int m = 0; m < 8; ++m) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                        }
+                    }
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                return;
+            }
+
 #pragma unroll
             for (int fj = 0; fj < kFragCols; ++fj)
                 b[0][fj] = fragment(buf + bOff[0] + fj * 16 * kRowBytes);
@@ -484,7 +548,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
                     }
-                    if (first && ks == 0) init_row(fi + 1);
+                    if (first && !kRowMajorFirstSlab && ks == 0) init_row(fi + 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -505,7 +569,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         acc[fi + 4][fj] =
                             __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
                     }
-                    if (first && ks == 0 && fi < 3) init_row(fi + 5);
+                    if (first && !kRowMajorFirstSlab && ks == 0 && fi < 3) init_row(fi + 5);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
