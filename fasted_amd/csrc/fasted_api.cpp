@@ -850,6 +850,32 @@ double search_epsilon(double targetSelectivity, double initialEpsilon, double* s
     return eps;
 }
 
+// Epsilon for a target selectivity by volume scaling (results/scripts/experiment/experiments.py:100-150,
+// 284-323): the number of neighbours is taken to grow like the volume of the epsilon ball, so a probe with
+// selectivity s at epsilon e predicts  e * (target / s)^(1/D)  -- the reference forms the two ball volumes with
+// pi^(D/2) / Gamma(D/2 + 1) in decimal arithmetic; the constants cancel -- and an empty probe doubles epsilon.
+// Ends within 10 % of the target, the reference's threshold for this search.  The reference's loop probes the
+// initial epsilon again instead of the adjusted one (experiments.py:314) and so never ends unless the first
+// probe is already close enough; here the adjusted epsilon is probed.
+template <typename Probe>
+double search_epsilon_volumetric(double targetSelectivity, double initialEpsilon, int dims, double* selectivity,
+                                 Probe&& probe) {
+    if (!(targetSelectivity > 0.0)) throw std::invalid_argument("target selectivity must be positive");
+    if (!(initialEpsilon > 0.0)) throw std::invalid_argument("initial epsilon must be positive");
+    if (dims < 1) throw std::invalid_argument("no resident dataset");
+    double eps = initialEpsilon, current = probe(eps);
+    int guard = 0;
+    while (!(std::fabs(current - targetSelectivity) / targetSelectivity < 0.1)) {
+        const double next = current == 0.0 ? eps * 2.0 : eps * std::pow(targetSelectivity / current, 1.0 / (double)dims);
+        if (++guard > 200 || next == eps || !std::isfinite(next))
+            throw std::runtime_error("volumetric epsilon search did not converge to within 10% of the target selectivity");
+        eps = next;
+        current = probe(eps);
+    }
+    if (selectivity) *selectivity = current;
+    return eps;
+}
+
 template <typename F>
 int guarded(F&& body) {
     try {
@@ -1048,6 +1074,20 @@ int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double*
         const int n = g_res.table.n;
         int count = 0;
         const double eps = search_epsilon(targetSelectivity, initialEpsilon, selectivity, [&](double e) {
+            ++count;
+            return selectivity_of(count_resident(e).pairsFound, n);
+        });
+        if (epsilon) *epsilon = eps;
+        if (probes) *probes = count;
+    });
+}
+
+int fasted_find_epsilon_volumetric(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
+                                   int* probes) {
+    return guarded([&] {
+        const int n = g_res.table.n;
+        int count = 0;
+        const double eps = search_epsilon_volumetric(targetSelectivity, initialEpsilon, g_res.table.d, selectivity, [&](double e) {
             ++count;
             return selectivity_of(count_resident(e).pairsFound, n);
         });

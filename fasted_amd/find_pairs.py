@@ -130,6 +130,9 @@ def load_findpairs(path: str = None):
                                                  c.c_void_p]
     lib.fasted_set_save_distances.restype = None
     lib.fasted_set_save_distances.argtypes = [c.c_int]
+    lib.fasted_find_epsilon_volumetric.restype = c.c_int
+    lib.fasted_find_epsilon_volumetric.argtypes = [c.c_double, c.c_double, c.POINTER(c.c_double), c.POINTER(c.c_double),
+                                                   c.POINTER(c.c_int)]
     lib.fasted_count_pairs_sampled.restype = c.c_int
     lib.fasted_count_pairs_sampled.argtypes = [c.c_double, c.c_int, c.POINTER(c.c_ulonglong), c.POINTER(c.c_int),
                                                c.POINTER(c.c_double)]
@@ -271,6 +274,16 @@ def find_epsilon(target_selectivity, initial_epsilon=0.0):
     eps, sel, probes = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
     _check(lib, lib.fasted_find_epsilon(float(target_selectivity), float(initial_epsilon), ctypes.byref(eps),
                                         ctypes.byref(sel), ctypes.byref(probes)))
+    return eps.value, sel.value, probes.value
+
+
+def find_epsilon_volumetric(target_selectivity, initial_epsilon=0.1):
+    """Native volume-scaling epsilon search on the resident dataset (within 10 % of the target, as the reference's
+    find_epsilon_volumetric): (epsilon, selectivity, probes)."""
+    lib = load_findpairs()
+    eps, sel, probes = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
+    _check(lib, lib.fasted_find_epsilon_volumetric(float(target_selectivity), float(initial_epsilon), ctypes.byref(eps),
+                                                   ctypes.byref(sel), ctypes.byref(probes)))
     return eps.value, sel.value, probes.value
 
 

@@ -217,6 +217,15 @@ int fasted_count_pairs(double epsilon, unsigned long long* pairsFound, double* k
 int fasted_find_epsilon(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
                         int* probes);
 
+/* Epsilon for a target selectivity by volume scaling, the reference's find_epsilon_volumetric with
+ * adjust_epsilon_volume (results/scripts/experiment/experiments.py:100-150,284-323): each count-only probe with
+ * selectivity s at epsilon e predicts e * (target / s)^(1/D), an empty probe doubles epsilon, the search ends
+ * within 10 % of the target.  `initialEpsilon` must be positive (the reference's default is 0.1).  The reference's
+ * loop probes the initial epsilon again instead of the adjusted one (experiments.py:314); the adjusted one is
+ * probed here.  Fails after 200 probes. */
+int fasted_find_epsilon_volumetric(double targetSelectivity, double initialEpsilon, double* epsilon, double* selectivity,
+                                   int* probes);
+
 /* The same probe and the same search on an evenly spaced sample of `sample_rows` query points against all
  * points (sample_rows/N of the work per probe): *pairsFound - *sampledRows estimates sampledRows x
  * selectivity.  fasted_find_epsilon_sampled runs the search of fasted_find_epsilon on sampled probes and

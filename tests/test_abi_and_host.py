@@ -296,6 +296,27 @@ def test_epsilon_search_restatement_follows_the_reference_procedure():
     assert calls == [2.0, 1.0, 0.5, 0.25]
 
 
+def test_volumetric_epsilon_search_restatement():
+    """The restated volume scaling against what the mathematics fixes: the constants of the two ball volumes
+    cancel, so a step is eps * (target / s)^(1/D); on a selectivity that is exactly c * eps^D one step lands on
+    the target; an empty probe doubles epsilon."""
+    from oracle import epsilon_search as ex
+
+    assert abs(float(ex.compute_gamma(4)) - 2.0) < 1e-12            # Gamma(3) = 2
+    assert abs(float(ex.compute_gamma(5)) - 3.323350970447843) < 1e-12  # Gamma(7/2) = 15 sqrt(pi) / 8
+    assert ex.adjust_epsilon_volume(0.3, 0, 10.0, 64) == 0.6
+    for eps, s, t, d in [(0.1, 3.0, 64.0, 2), (2.5, 1000.0, 16.0, 128), (0.03, 0.5, 200.0, 4096), (7.0, 9.0, 9.5, 17)]:
+        assert abs(ex.adjust_epsilon_volume(eps, s, t, d) / (eps * (t / s) ** (1.0 / d)) - 1.0) < 1e-12
+    calls = []
+    eps = ex.find_epsilon_volumetric(3, 64.0, lambda e: calls.append(e) or 700.0 * e ** 3)
+    assert len(calls) == 2 and calls[0] == 0.1 and abs(700.0 * eps ** 3 - 64.0) < 1e-9
+    calls = []
+    eps = ex.find_epsilon_volumetric(8, 5.0, lambda e: calls.append(e) or (0.0 if e < 0.35 else 40.0 * e ** 2))
+    assert calls[:3] == [0.1, 0.2, 0.4] and ex.within_percent(40.0 * eps ** 2, 5.0, 0.1)
+    with pytest.raises(RuntimeError):
+        ex.find_epsilon_volumetric(2, 5.0, lambda e: 1.0, max_iterations=20)  # a plateau never gets there
+
+
 def test_pair_statistics_and_per_point_iou():
     from fasted_amd import accuracy as ex
 

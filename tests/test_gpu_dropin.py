@@ -119,6 +119,34 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     lib.releaseResources()
 
 
+def test_native_volumetric_epsilon_search(lib):
+    """fasted_find_epsilon_volumetric against the restated procedure driven by count-only probes: the same
+    probes (the decimal and the double form of a step agree to rounding), an epsilon within 10 % of the target."""
+    import ctypes
+
+    import fasted_amd
+    from oracle import epsilon_search as ex
+
+    n, d = 6000, 64
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    eps, sel, probes = fasted_amd.find_epsilon_volumetric(16.0, 0.1)
+    assert ex.within_percent(sel, 16.0, 0.1) and probes >= 2
+    calls = []
+
+    def get_selectivity(e):
+        calls.append(e)
+        return fasted_amd.compute_selectivity(fasted_amd.count_pairs(e)[0], n)
+
+    want = ex.find_epsilon_volumetric(d, 16.0, get_selectivity, 0.1)
+    assert len(calls) == probes and abs(want - eps) <= 1e-9 * eps
+    assert fasted_amd.compute_selectivity(fasted_amd.count_pairs(eps)[0], n) == sel
+    # bad arguments come back as errors, not as a loop
+    e, s_, p_ = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
+    assert lib.fasted_find_epsilon_volumetric(16.0, 0.0, ctypes.byref(e), ctypes.byref(s_), ctypes.byref(p_)) != 0
+    assert lib.fasted_find_epsilon_volumetric(-1.0, 0.1, ctypes.byref(e), ctypes.byref(s_), ctypes.byref(p_)) != 0
+    lib.releaseResources()
+
+
 def test_sampled_epsilon_search(lib):
     """The search on sampled probes: the sampled count equals the count of the same rows in the full pair
     list, and the epsilon found lands close to the full search's at a fraction of the work."""
