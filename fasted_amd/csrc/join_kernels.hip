@@ -650,14 +650,20 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 any = __builtin_amdgcn_ballot_w64(best >= 0.0f) != 0ull;
                 if (any) {
                     // the rows of blocks with a hit somewhere in the wave yield their bits, one instruction per
-                    // element: the sign of the accumulator (set = no hit) is shifted in
+                    // element: the sign of the accumulator (set = no hit) is shifted in.  (The eight compares are
+                    // issued together: one at a time, each branch waits for its compare.)
+                    unsigned long long rowHit[kFragRows];
+#pragma unroll
+                    for (int fi = 0; fi < kFragRows; ++fi) rowHit[fi] = __builtin_amdgcn_ballot_w64(rowBest[fi] >= 0.0f);
+#pragma unroll
+                    for (int fi = 0; fi < kFragRows; ++fi) asm volatile("" : "+s"(rowHit[fi]));
 #pragma unroll
                     for (int fp = 0; fp < kFragRows / 2; ++fp) {
                         unsigned m = ~0u;
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
                             const int fi = fp * 2 + h;
-                            if (__builtin_amdgcn_ballot_w64(rowBest[fi] >= 0.0f) != 0ull) {
+                            if (rowHit[fi] != 0ull) {
 #pragma unroll
                                 for (int fj = 0; fj < kFragCols; ++fj)
 #pragma unroll
@@ -695,41 +701,57 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 }
             }
             if (any) {
-                // Extraction, one word of hit bits after the other.  Each round takes the first remaining hit
-                // of every lane that has one: the lanes form a mask in scalar registers, a lane's record goes
-                // behind those of the lanes before it, the wave's fill count moves on by the number of lanes.
-#pragma unroll
-                for (int fp = 0; fp < kFragRows / 2; ++fp) {
-                    unsigned w = hits[fp];
-                    for (;;) {
-                        const unsigned long long lanes = __builtin_amdgcn_ballot_w64(w != 0u);
-                        if (lanes == 0ull) break;
-                        const int count = __builtin_popcountll(lanes) << (mirror ? 1 : 0);
-                        if (staged + count > kWaveStagePairs) flush_wave();
-                        if (w != 0u) {
-                            const int e = __builtin_clz(w);  // element number inside the pair of block rows
-                            w &= ~(0x80000000u >> e);
-                            const int q = qLane + fp * 32 + (e >> 4) * 16 + (e & 3);
-                            const int c = cLane + ((e >> 2) & 3) * 16;
-                            const unsigned before = __builtin_amdgcn_mbcnt_hi(
-                                (unsigned)(lanes >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)lanes, 0u));
-                            const unsigned at = (unsigned)staged + (mirror ? 2u * before : before);
-                            // written as an instruction: for an ordinary LDS store the compiler first waits until
-                            // this wave's global->LDS transfers of the next tile have landed
-                            auto put = [&](unsigned idx, int first, int second) {
-                                const unsigned long long rec =
-                                    (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
-                                asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage +
-                                                                         ((unsigned)wave * kWaveStagePairs + idx) * 8u),
-                                             "v"(rec)
-                                             : "memory");
-                            };
-                            put(at, q, c);
-                            if (mirror) put(at + 1, c, q);
-                        }
-                        staged += count;
+                // Extraction.  A round takes the first remaining hit of every lane that has one in a word of hit
+                // bits: the lanes form a mask in scalar registers, a lane's record goes behind those of the lanes
+                // before it, the wave's fill count moves on by the number of lanes.
+                auto take_round = [&](int fp, unsigned long long lanes) {
+                    const int count = __builtin_popcountll(lanes) << (mirror ? 1 : 0);
+                    if (staged + count > kWaveStagePairs) flush_wave();
+                    unsigned& w = hits[fp];
+                    if (w != 0u) {
+                        const int e = __builtin_clz(w);  // element number inside the pair of block rows
+                        w &= ~(0x80000000u >> e);
+                        const int q = qLane + fp * 32 + (e >> 4) * 16 + (e & 3);
+                        const int c = cLane + ((e >> 2) & 3) * 16;
+                        const unsigned before = __builtin_amdgcn_mbcnt_hi(
+                            (unsigned)(lanes >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)lanes, 0u));
+                        const unsigned at = (unsigned)staged + (mirror ? 2u * before : before);
+                        // written as an instruction: for an ordinary LDS store the compiler first waits until
+                        // this wave's global->LDS transfers of the next tile have landed
+                        auto put = [&](unsigned idx, int first, int second) {
+                            const unsigned long long rec =
+                                (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
+                            asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage +
+                                                                     ((unsigned)wave * kWaveStagePairs + idx) * 8u),
+                                         "v"(rec)
+                                         : "memory");
+                        };
+                        put(at, q, c);
+                        if (mirror) put(at + 1, c, q);
                     }
-                }
+                    staged += count;
+                };
+                // The four words' masks are formed together, and again together after every word has had a round
+                // (a branch on a mask waits for the compare that forms it: one at a time, that wait is paid per
+                // word and round; most lanes have one hit at most, so the second set of masks is usually empty).
+                unsigned long long lanes[kFragRows / 2];
+                auto form_masks = [&]() {
+#pragma unroll
+                    for (int fp = 0; fp < kFragRows / 2; ++fp) lanes[fp] = __builtin_amdgcn_ballot_w64(hits[fp] != 0u);
+#pragma unroll
+                    for (int fp = 0; fp < kFragRows / 2; ++fp) asm volatile("" : "+s"(lanes[fp]));
+                };
+                form_masks();
+#pragma unroll
+                for (int fp = 0; fp < kFragRows / 2; ++fp)
+                    if (lanes[fp] != 0ull) take_round(fp, lanes[fp]);
+                form_masks();
+#pragma unroll
+                for (int fp = 0; fp < kFragRows / 2; ++fp)
+                    while (lanes[fp] != 0ull) {
+                        take_round(fp, lanes[fp]);
+                        lanes[fp] = __builtin_amdgcn_ballot_w64(hits[fp] != 0u);
+                    }
             }
         } else {
             // keep the accumulators observable without spending instructions on them
