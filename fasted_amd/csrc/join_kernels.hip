@@ -26,6 +26,7 @@
 // tile before its result is used, and the optimiser's wave-reduction form would wait for it on the spot.
 #include "join_kernels.h"
 
+#include <cstdlib>
 #include <type_traits>
 
 #include "join_device.hpp"
@@ -46,7 +47,7 @@ constexpr int kLdsStage = kLdsNext + 16;            // staged pairs: one private
 constexpr int kWaveStagePairs = 384;                // 3 KiB of 8-byte records per wave
 constexpr int kLdsBytes = kLdsStage + 8 * kWaveStagePairs * 8;
 static_assert(kLdsBytes <= 160 * 1024, "LDS budget of one CU");
-constexpr int kWaveRows = 128, kWaveCols = 64;      // output sub-tile of one wave
+constexpr int kWaveCols = 64;                       // columns of a wave's output sub-tile (its rows: half the tile's)
 
 // Measurement builds (`make ablation`): the join kernel with parts compiled out, to see what each part
 // costs in time and in power.  Such a build computes wrong results; the library proper is built with 0.
@@ -75,11 +76,7 @@ __device__ __forceinline__ half8 fragment(const unsigned char* p) {
     }
     return *reinterpret_cast<const half8*>(p);
 }
-#ifndef FASTED_ROW_MAJOR_FIRST_SLAB
-#define FASTED_ROW_MAJOR_FIRST_SLAB 1
-#endif
-constexpr bool kRowMajorFirstSlab = FASTED_ROW_MAJOR_FIRST_SLAB != 0;
-constexpr int kFragRows = kWaveRows / 16, kFragCols = kWaveCols / 16;  // 8 x 4 MFMA 16x16 blocks
+constexpr int kFragCols = kWaveCols / 16;  // a wave's sub-tile: 8 (or 4) x 4 MFMA 16x16 blocks
 
 // Operand rows of the 256x256 kernel are 128 bytes (a 64-wide k-slab): see lds_swizzle128 in
 // tile_order.hpp (conflict freedom is checked exhaustively on the host by tests, and with the
@@ -104,14 +101,14 @@ struct SubShape {
     static constexpr int rows = kTall ? 8 : 4, cols = kTall ? 4 : 8;
 };
 
-inline bool tall_order(long long nQueries) {
-    return (nQueries + kTile - 1) / kTile >= 64;
+inline bool tall_order(long long nQueries, int tileRows = kTile) {
+    return (nQueries + tileRows - 1) / tileRows >= 64;
 }
 
-inline Raster make_raster(long long nQueries, long long nCandidates, bool upperOnly = false) {
-    const bool tall = tall_order(nQueries);
-    return tall ? make_tile_order(nQueries, nCandidates, kTile, kTile, SubShape<true>::rows, SubShape<true>::cols, upperOnly)
-                : make_tile_order(nQueries, nCandidates, kTile, kTile, SubShape<false>::rows, SubShape<false>::cols, upperOnly);
+inline Raster make_raster(long long nQueries, long long nCandidates, bool upperOnly = false, int tileRows = kTile) {
+    const bool tall = tall_order(nQueries, tileRows);
+    return tall ? make_tile_order(nQueries, nCandidates, tileRows, kTile, SubShape<true>::rows, SubShape<true>::cols, upperOnly)
+                : make_tile_order(nQueries, nCandidates, tileRows, kTile, SubShape<false>::rows, SubShape<false>::cols, upperOnly);
 }
 
 // host mirror of the kernels' decoding
@@ -238,8 +235,16 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-template <bool kEpilogue, bool kTall>
+// kTileRows = 256, or 128 for matrices of few tiles: the tile grid is then twice as fine along the queries (a wave's
+// sub-tile is 64 x 64, 4 x 4 blocks), so that twice as many workgroups find work.  The transfers stay as they
+// are -- 256 query rows from the tile's first row on are staged, the lower half unused -- which costs nothing
+// that matters at such sizes and keeps one set of addresses.
+template <bool kEpilogue, bool kTall, int kTileRows>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
+    static_assert(kTileRows == 256 || kTileRows == 128, "tile rows");
+    constexpr int kWaveRows = kTileRows / 2;    // rows of a wave's output sub-tile (2 x 4 waves)
+    constexpr int kFragRows = kWaveRows / 16;   // its rows of 16x16 blocks
+    constexpr int kHalfRows = kFragRows / 2;    // a k-step goes through them in two halves
     __shared__ __align__(16) unsigned char lds[kLdsBytes];
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);  // wave-uniform, lives in an SGPR
     const int wr = wave >> 2, wc = wave & 3;
@@ -398,8 +403,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __syncthreads();  // everybody has read sNext before thread 0 writes the second tile there
 
     unsigned offA[4], offB[4];
-    tile_offsets((int)tr * kTile, (int)tc * kTile, offA, offB, true);
-    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(tr) * kTile * p.ldQ16);
+    tile_offsets((int)tr * kTileRows, (int)tc * kTile, offA, offB, true);
+    const char* gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(tr) * kTileRows * p.ldQ16);
     const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(tc) * kTile * p.ldC16);
     static_for<0, 8>([&](auto jc) { issue_load(jc, gA, gB, offA, offB, 0); });
     if (kNoTransfers) {
@@ -407,7 +412,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         static_for<0, 8>([&](auto jc) { issue_load(jc, gA + second, gB + second, offA, offB, 1); });
         filling = false;
     }
-    issue_sums((int)tr * kTile, (int)tc * kTile, 0);
+    issue_sums((int)tr * kTileRows, (int)tc * kTile, 0);
     unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
     if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
 
@@ -466,9 +471,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                              const unsigned (&oA)[4], const unsigned (&oB)[4]) {
             constexpr bool first = decltype(firstc)::value;  // the tile's first slab also sets the accumulators
             const unsigned char* const buf = lds + stg * kStageBytes;
-            half8 aLo[4], aHi[4], b[2][kFragCols];
+            half8 aLo[kHalfRows], aHi[kHalfRows], b[2][kFragCols];
 
-            if constexpr (first && kRowMajorFirstSlab) {
+            if constexpr (first) {
                 // The tile's first slab goes through the rows of blocks one after the other, both k-steps of a
                 // row together (an element still receives k-step 0 before k-step 1): the 16 start values of row
                 // fi + 1 are formed between the 8 MFMAs of row fi, two vector instructions behind every MFMA,
@@ -532,23 +537,22 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             for (int fj = 0; fj < kFragCols; ++fj)
                 b[0][fj] = fragment(buf + bOff[0] + fj * 16 * kRowBytes);
 #pragma unroll
-            for (int fi = 0; fi < 4; ++fi)
+            for (int fi = 0; fi < kHalfRows; ++fi)
                 aLo[fi] = fragment(buf + aOff[0] + fi * 16 * kRowBytes);
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-                for (int fi = 0; fi < 4; ++fi)
-                    aHi[fi] = fragment(buf + aOff[ks] + (fi + 4) * 16 * kRowBytes);
+                for (int fi = 0; fi < kHalfRows; ++fi)
+                    aHi[fi] = fragment(buf + aOff[ks] + (fi + kHalfRows) * 16 * kRowBytes);
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0 && prefetch) static_for<0, 4>([&](auto jc) { issue_load(jc, pA, pB, oA, oB, stg ^ 1); });
 #pragma unroll
-                for (int fi = 0; fi < 4; ++fi) {
+                for (int fi = 0; fi < kHalfRows; ++fi) {
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;  // snake order: one operand in common with the MFMA before
                         acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aLo[fi], b[ks][fj], acc[fi][fj], 0, 0, 0);
                     }
-                    if (first && !kRowMajorFirstSlab && ks == 0) init_row(fi + 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0) {
@@ -556,20 +560,19 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                     for (int fj = 0; fj < kFragCols; ++fj)
                         b[1][fj] = fragment(buf + bOff[1] + fj * 16 * kRowBytes);
 #pragma unroll
-                    for (int fi = 0; fi < 4; ++fi)
+                    for (int fi = 0; fi < kHalfRows; ++fi)
                         aLo[fi] = fragment(buf + aOff[1] + fi * 16 * kRowBytes);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks == 0 && prefetch) static_for<4, 8>([&](auto jc) { issue_load(jc, pA, pB, oA, oB, stg ^ 1); });
 #pragma unroll
-                for (int fi = 0; fi < 4; ++fi) {
+                for (int fi = 0; fi < kHalfRows; ++fi) {
 #pragma unroll
                     for (int fs = 0; fs < kFragCols; ++fs) {
                         const int fj = (fi & 1) ? kFragCols - 1 - fs : fs;
-                        acc[fi + 4][fj] =
-                            __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + 4][fj], 0, 0, 0);
+                        acc[fi + kHalfRows][fj] =
+                            __builtin_amdgcn_mfma_f32_16x16x32_f16(aHi[fi], b[ks][fj], acc[fi + kHalfRows][fj], 0, 0, 0);
                     }
-                    if (first && !kRowMajorFirstSlab && ks == 0 && fi < 3) init_row(fi + 5);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -596,10 +599,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         const unsigned ntc = __builtin_amdgcn_readfirstlane(sNext[1]);
         const bool more = ntr != kNoTile;
         if (more) {
-            tile_offsets((int)ntr * kTile, (int)ntc * kTile, offA, offB, false);
-            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(ntr) * kTile * p.ldQ16);
+            tile_offsets((int)ntr * kTileRows, (int)ntc * kTile, offA, offB, false);
+            gA = reinterpret_cast<const char*>(p.ptsQ + (long long)panel_of(ntr) * kTileRows * p.ldQ16);
             gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(ntc) * kTile * p.ldC16);
-            issue_sums((int)ntr * kTile, (int)ntc * kTile, sumsBuf ^ 1);
+            issue_sums((int)ntr * kTileRows, (int)ntc * kTile, sumsBuf ^ 1);
         }
         if (p.nSlabs == 1) {  // a single slab: all rows are set before it
 #pragma unroll
@@ -613,7 +616,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             // h = eps^2/4 - s/2 per point, so an element now holds a = q.c - (s_q + s_c)/2 + eps^2/2 =
             // (eps^2 - dist^2)/2 and the reference's test  s_q + s_c - 2 q.c <= eps^2  reads  a >= 0: the sign
             // bit of the accumulator, symmetric in q and c like the reference's test.
-            const int rowBase = (int)tr * kTile, colBase = (int)tc * kTile;
+            const int rowBase = (int)tr * kTileRows, colBase = (int)tc * kTile;
             const int ln = lane_now();
             const int qLane = rowBase + wr * kWaveRows + (ln >> 4) * 4;  // row of element r = 0 of block row 0
             const int cLane = colBase + wc * kWaveCols + (ln & 15);      // column in block column 0
@@ -622,9 +625,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             // or when the dataset holds points with non-finite norms (a NaN must compare as "no hit").
             // (forced pairs: query q with candidate q * selfStride -- the diagonal of a self-join, or the sampled
             // points among all points)
-            const bool diagonal = p.selfStride != 0 && colBase <= (rowBase + kTile - 1) * p.selfStride &&
+            const bool diagonal = p.selfStride != 0 && colBase <= (rowBase + kTileRows - 1) * p.selfStride &&
                                   rowBase * p.selfStride <= colBase + kTile - 1;
-            const bool edge = nonFinite || diagonal || rowBase + kTile > p.nQ || colBase + kTile > p.nC;
+            const bool edge = nonFinite || diagonal || rowBase + kTileRows > p.nQ || colBase + kTile > p.nC;
             const bool mirror = p.symmetric && tr != tc;  // a tile above the diagonal also stands for its mirror image
 
             // Per-lane hit bits of the 4 pairs of block rows: element e = (fi & 1) * 16 + fj * 4 + r of the pair
@@ -895,21 +898,35 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     p.counters = l.counters;
     p.pairs = static_cast<int2*>(l.pairs);
     p.cap = l.cap;
-    p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0);
+    // Tiles of 128 query rows when the matrix has too few 256 x 256 tiles to occupy the chip (never in symmetric
+    // mode, whose diagonal logic assumes square tiles).  A 128-row tile costs about 0.7 of a 256-row one (64 x 64
+    // wave sub-tiles need a third more LDS fragment reads per MFMA), so the finer grid only pays while the coarse
+    // one leaves a good part of the workgroups idle: measured on Exp(40) data, 2154 points 1.1x (D = 128) to 1.5x
+    // (D = 4096) faster, 3000 points 1.1x, from 4096 points (256 tiles, one per CU) on slower.
+    // FASTED_TILE_ROWS=256 or 128 in the environment overrides the choice (tests run both).
+    const unsigned long long tiles256 = (unsigned long long)((l.nQ + kTile - 1) / kTile) * ((l.nC + kTile - 1) / kTile);
+    bool rows128 = p.symmetric == 0 && tiles256 * 5ull <= 3ull * (unsigned long long)numCUs;
+    const char* const forced = getenv("FASTED_TILE_ROWS");  // read at every launch: a test sets it per case
+    const int forcedRows = forced ? atoi(forced) : 0;
+    if (forcedRows == 256) rows128 = false;
+    if (forcedRows == 128 && p.symmetric == 0) rows128 = true;
+    const int tileRows = rows128 ? 128 : kTile;
+    p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0, tileRows);
     unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
     unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
-    const bool tall = tall_order(l.nQ);
-    if (l.epilogue) {
-        if (tall)
-            join_kernel<true, true><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
-        else
-            join_kernel<true, false><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
-    } else {
-        if (tall)
-            join_kernel<false, true><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
-        else
-            join_kernel<false, false><<<dim3(grid), dim3(kThreads), 0, stream>>>(p);
+    const bool tall = tall_order(l.nQ, tileRows);
+    const dim3 g(grid), b(kThreads);
+    const int variant = (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
+    switch (variant) {
+        case 7: join_kernel<true, true, 128><<<g, b, 0, stream>>>(p); break;
+        case 6: join_kernel<true, true, 256><<<g, b, 0, stream>>>(p); break;
+        case 5: join_kernel<true, false, 128><<<g, b, 0, stream>>>(p); break;
+        case 4: join_kernel<true, false, 256><<<g, b, 0, stream>>>(p); break;
+        case 3: join_kernel<false, true, 128><<<g, b, 0, stream>>>(p); break;
+        case 2: join_kernel<false, true, 256><<<g, b, 0, stream>>>(p); break;
+        case 1: join_kernel<false, false, 128><<<g, b, 0, stream>>>(p); break;
+        default: join_kernel<false, false, 256><<<g, b, 0, stream>>>(p); break;
     }
     return hipGetLastError();
 }

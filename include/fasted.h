@@ -76,7 +76,8 @@ typedef struct FastedJoinStats {
     float sortMs;       /* host wall time of the row-major sort, stream synchronisation included (0 when not sorted) */
     int paddedN;        /* rows covered by the tile grid */
     int paddedD;        /* K extent the kernel looped over */
-    unsigned long long tiles;      /* 256x256 tiles computed (with FASTED_SYMMETRIC: those on and above the diagonal) */
+    unsigned long long tiles;      /* size of the distance matrix in 256x256 tiles (with FASTED_SYMMETRIC: those on and
+                                      above the diagonal); small matrices are computed in 128x256 tiles, two per unit */
     unsigned long long pairsFound;
     unsigned long long pairsStored;
 } FastedJoinStats;

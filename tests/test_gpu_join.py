@@ -435,3 +435,39 @@ def test_tall_tile_order_exact_pair_sets(fasted):
     st = fasted.join_device(pts.data_ptr(), n, d, pts.data_ptr(), nc, d, d, eps, pairs.data_ptr(), pairs.shape[0])
     assert st.pairsFound == st.pairsStored == want2.shape[0]
     assert bool((pairs[: st.pairsStored] == want2).all())
+
+
+@pytest.mark.parametrize("n,d", [(300, 64), (1025, 192), (2154, 128), (4642, 64), (64 * 128 + 37, 64)])
+def test_both_tile_heights_give_the_exact_pair_set(fasted, n, d, monkeypatch):
+    """Matrices of few tiles are cut into tiles of 128 query rows instead of 256 (FASTED_TILE_ROWS forces either).
+    Integer coordinates make the join exact: both heights, on a self-join, on a two-set join with a ragged
+    query count and with non-finite points present, must give exactly the FP64 pair list.  The last shape has
+    65 tile rows of 128: the tall tile order with that height."""
+    import torch
+
+    bits = datasets.small_integers(n, d, high=3, seed=3 * n + d)
+    x = bits.view(np.float16).astype(np.float64)
+    d2 = ((x[:64, None, :] - x[None, :64, :]) ** 2).sum(-1)
+    eps = float(np.sqrt(np.sort(d2[np.triu_indices(64, 1)])[40] + 0.5))
+    truth = oracle.self_join_f64(bits, eps)
+    nq = n - 131  # a ragged query set against the first 700 points (or all of them)
+    nc = min(n, 700)
+    truth2 = truth[(truth[:, 0] < nq) & (truth[:, 1] < nc)]
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    for rows in ("256", "128"):
+        monkeypatch.setenv("FASTED_TILE_ROWS", rows)
+        got, st, _ = device_join(fasted, bits, eps)
+        assert st.pairsFound == len(truth) and np.array_equal(got, truth), rows
+        buf = torch.empty((len(truth2) + 64, 2), dtype=torch.int32, device="cuda")
+        st2 = fasted.join_device(pts.data_ptr(), nq, d, pts.data_ptr(), nc, d, d, eps, buf.data_ptr(), buf.shape[0])
+        assert st2.pairsFound == len(truth2) and np.array_equal(buf[: st2.pairsStored].cpu().numpy(), truth2), rows
+    # a point with an infinite coordinate pairs with nothing but itself, under both heights
+    bad = bits.copy()
+    bad[5, 0] = 0x7C00
+    keep = truth[(truth[:, 0] != 5) & (truth[:, 1] != 5)]
+    want = np.concatenate([keep, np.array([[5, 5]], dtype=np.int32)])
+    want = want[np.lexsort((want[:, 1], want[:, 0]))]
+    for rows in ("256", "128"):
+        monkeypatch.setenv("FASTED_TILE_ROWS", rows)
+        got, st, _ = device_join(fasted, bad, eps)
+        assert np.array_equal(got, want), rows

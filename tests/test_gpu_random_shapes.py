@@ -18,9 +18,15 @@ def cases(count=48, seed=2024):
             for _ in range(count)]
 
 
+@pytest.mark.parametrize("tile_rows", ["auto", "256", "128"])  # the library's choice, then each tile height forced
 @pytest.mark.parametrize("n,d,neighbours,seed", cases())
-def test_random_shape(n, d, neighbours, seed):
+def test_random_shape(n, d, neighbours, seed, tile_rows, monkeypatch):
     import torch
+
+    if tile_rows == "auto":
+        monkeypatch.delenv("FASTED_TILE_ROWS", raising=False)
+    else:
+        monkeypatch.setenv("FASTED_TILE_ROWS", tile_rows)
 
     import fasted_amd
     from fasted_amd import find_pairs as fp
