@@ -27,6 +27,7 @@ struct JoinParams {
     int selfStride;  // != 0: (q, q * selfStride) is always a pair -- 1 for a self-join ((i, i) is a pair)
     int symmetric; // self-join only: compute tiles on and above the diagonal, emit (q,c) and (c,q)
     int nSlabs;    // 64-wide k-slabs per tile
+    int direct;    // != 0: no more tiles than workgroups: workgroup b computes tile b and nothing else (no queues)
     const float* halfQ;  // per query point: eps^2/4 - s/2, s = squared norm
     const float* halfC;  // ... per candidate point
     unsigned long long* counters;

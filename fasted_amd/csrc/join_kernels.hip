@@ -392,7 +392,16 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // ---- first tile
     if (wave == 0 && lane_now() == 0) {
         unsigned r, c;
-        find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r, &c);
+        if (p.direct) {
+            // A matrix of no more tiles than workgroups: one tile each, by workgroup number.  Through the queues,
+            // every workgroup would reserve a second tile while it starts its first (the reservation runs one
+            // tile ahead), and the workgroups of XCDs with short queues would find the work already taken.
+            r = blockIdx.x / p.raster.tileCols;
+            c = blockIdx.x % p.raster.tileCols;
+            if (p.symmetric && c < r) r = kNoTile;
+        } else {
+            find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r, &c);
+        }
         sNext[0] = r;
         sNext[1] = c;
     }
@@ -414,7 +423,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     }
     issue_sums((int)tr * kTileRows, (int)tc * kTile, 0);
     unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
-    if (wave == 0 && lane_now() == 0) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
+    if (wave == 0 && lane_now() == 0 && !p.direct) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
 
     int stage = 0;  // LDS stage that holds slab 0 of the current tile
     int sumsBuf = 0;
@@ -425,10 +434,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         if (wave == 0 && lane_now() == 0) {
             // the reservation made a whole tile ago has long arrived: no wait here
             unsigned r, c;
-            find_tile(popped, &r, &c);
+            if (p.direct) {
+                r = kNoTile;
+                c = 0u;
+            } else {
+                find_tile(popped, &r, &c);
+                popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
+            }
             sNext[0] = r;
             sNext[1] = c;
-            popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
         }
 
         // The accumulators start at h_q + h_c, h = eps^2/4 - s/2 per point (see the epilogue): the tile's
@@ -898,14 +912,14 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     p.counters = l.counters;
     p.pairs = static_cast<int2*>(l.pairs);
     p.cap = l.cap;
-    // Tiles of 128 query rows when the matrix has too few 256 x 256 tiles to occupy the chip (never in symmetric
-    // mode, whose diagonal logic assumes square tiles).  A 128-row tile costs about 0.7 of a 256-row one (64 x 64
-    // wave sub-tiles need a third more LDS fragment reads per MFMA), so the finer grid only pays while the coarse
-    // one leaves a good part of the workgroups idle: measured on Exp(40) data, 2154 points 1.1x (D = 128) to 1.5x
-    // (D = 4096) faster, 3000 points 1.1x, from 4096 points (256 tiles, one per CU) on slower.
+    // Tiles of 128 query rows when the matrix then still has no more tiles than the chip has workgroups (never
+    // in symmetric mode, whose diagonal logic assumes square tiles): twice as many workgroups work, each on half a
+    // tile.  A 128-row tile costs about 0.7 of a 256-row one (64 x 64 wave sub-tiles need a third more LDS fragment
+    // reads per MFMA), so the finer grid only pays while it fits one round: measured on Exp(40) data, 1000 and 2154
+    // points 1.1x - 1.4x faster, 3000 points (288 tiles of 128 rows: two rounds) 1.4x slower.
     // FASTED_TILE_ROWS=256 or 128 in the environment overrides the choice (tests run both).
-    const unsigned long long tiles256 = (unsigned long long)((l.nQ + kTile - 1) / kTile) * ((l.nC + kTile - 1) / kTile);
-    bool rows128 = p.symmetric == 0 && tiles256 * 5ull <= 3ull * (unsigned long long)numCUs;
+    const unsigned long long tiles128 = (unsigned long long)((l.nQ + 127) / 128) * ((l.nC + kTile - 1) / kTile);
+    bool rows128 = p.symmetric == 0 && tiles128 <= (unsigned long long)numCUs;
     const char* const forced = getenv("FASTED_TILE_ROWS");  // read at every launch: a test sets it per case
     const int forcedRows = forced ? atoi(forced) : 0;
     if (forcedRows == 256) rows128 = false;
@@ -915,6 +929,7 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
     unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
+    p.direct = realTiles <= (unsigned long long)numCUs ? 1 : 0;  // grid == realTiles then: workgroup b takes tile b
     const bool tall = tall_order(l.nQ, tileRows);
     const dim3 g(grid), b(kThreads);
     const int variant = (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);

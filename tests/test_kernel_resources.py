@@ -43,7 +43,7 @@ def test_join_kernels_use_no_scratch_and_fit_one_cu():
         assert r["VGPRs Spill"] == 0, (name, r)
         # scalar registers that do not fit are parked in lanes of a vector register, not in memory: harmless in
         # small numbers (each costs a vector instruction where it is used)
-        assert r["SGPRs Spill"] <= 8, (name, r)
+        assert r["SGPRs Spill"] <= 12, (name, r)
         assert r["VGPRs"] + r["AGPRs"] <= 256, (name, r)  # two waves per SIMD
         assert r["Occupancy"] >= 2, (name, r)
         assert 0 < r["LDS Size"] <= LDS_PER_CU, (name, r)
