@@ -927,9 +927,11 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     const int tileRows = rows128 ? 128 : kTile;
     p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0, tileRows);
     unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
-    unsigned grid = (unsigned)(realTiles < (unsigned long long)numCUs ? realTiles : (unsigned long long)numCUs);
+    // Up to two tiles per CU, workgroup b computes tile b and ends, one workgroup per tile (the hardware places
+    // the second round as CUs fall free); from there on, one persistent workgroup per CU draws from the queues.
+    p.direct = realTiles <= 2ull * (unsigned long long)numCUs ? 1 : 0;
+    unsigned grid = (unsigned)(p.direct ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
-    p.direct = realTiles <= (unsigned long long)numCUs ? 1 : 0;  // grid == realTiles then: workgroup b takes tile b
     const bool tall = tall_order(l.nQ, tileRows);
     const dim3 g(grid), b(kThreads);
     const int variant = (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
