@@ -15,6 +15,8 @@ from .find_pairs import (  # noqa: F401
     count_pairs,
     find_epsilon,
     find_epsilon_sampled,
+    last_pairs_device,
+    set_download_pairs,
     find_epsilon_volumetric,
     join_device,
     library_path,
@@ -30,6 +32,6 @@ from .find_pairs import (  # noqa: F401
 )
 
 __all__ = [
-    "FastedJoinStats", "FastedPair", "check_padding_device", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "find_epsilon_sampled", "find_epsilon_volumetric", "join_device", "library_path",
+    "FastedJoinStats", "FastedPair", "check_padding_device", "RerunnablePairsFinder", "Results", "compute_selectivity", "count_pairs", "find_epsilon", "find_epsilon_sampled", "last_pairs_device", "set_download_pairs", "find_epsilon_volumetric", "join_device", "library_path",
     "load_findpairs", "mmaShape", "pair_distances_device", "resident_points", "self_join", "self_join_blocked", "self_join_device", "self_join_device_noalloc", "sum_squared_device",
 ]

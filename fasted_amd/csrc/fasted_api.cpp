@@ -468,6 +468,16 @@ std::string output_dir() {
 }
 
 bool g_saveDistances = false;
+bool g_downloadPairs = true;
+unsigned long long g_lastStored = 0;  // pairs the last resident run left, sorted, in the device pair buffer
+
+// The reference always copies the pair list to the host, saved or not (source/findPairs.cuh:711-713).  A caller
+// that only wants the counts, or goes on working with the pairs on the device, switches that off.
+bool download_pairs() {
+    if (!g_downloadPairs) return false;
+    const char* v = std::getenv("FASTED_DOWNLOAD_PAIRS");
+    return !(v && v[0] == '0');
+}
 
 bool save_distances() {
     if (g_saveDistances) return true;
@@ -666,8 +676,10 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
         HIP_CHECK(hipStreamSynchronize(nullptr));
     }
 
-    // The pairs always leave the device, saved or not (source/findPairs.cuh:705-714): piece by piece through
-    // two pinned buffers, the next piece travelling while the current one is written as text.
+    g_lastStored = st.pairsStored;
+    // The pairs leave the device, saved or not (source/findPairs.cuh:705-714; unless the caller has switched the
+    // download off and does not save): piece by piece through two pinned buffers, the next piece travelling while
+    // the current one is written as text.
     std::unique_ptr<PairsTextFile> file;
     if (savePairs) {
         const std::string path = output_dir() + "/" + datasetName + "_" + std::to_string(epsilon) + ".pairs";
@@ -675,7 +687,7 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
         file.reset(new PairsTextFile(path));
     }
     const size_t piece = PairWorkspace::kPiecePairs;
-    const size_t total = (size_t)st.pairsStored;
+    const size_t total = (savePairs || download_pairs()) ? (size_t)st.pairsStored : 0;
     auto fetch = [&](size_t first, int slot) {
         const size_t count = std::min(piece, total - first);
         HIP_CHECK(hipMemcpyAsync(g_pairWs.hPairs[slot], static_cast<const FastedPair*>(dPairs) + first,
@@ -1153,6 +1165,13 @@ const uint16_t* fasted_resident_points(int* n, int* d, int* n_pad, int* d_pad) {
 void fasted_set_output_dir(const char* dir) { g_outDir = dir ? dir : ""; }
 
 void fasted_set_save_distances(int enabled) { g_saveDistances = enabled != 0; }
+
+void fasted_set_download_pairs(int enabled) { g_downloadPairs = enabled != 0; }
+
+const FastedPair* fasted_last_pairs_device(unsigned long long* stored) {
+    if (stored) *stored = g_pairWs.dPairs ? g_lastStored : 0;
+    return static_cast<const FastedPair*>(g_pairWs.dPairs);
+}
 
 const char* fasted_last_error(void) { return g_error.c_str(); }
 

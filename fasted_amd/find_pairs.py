@@ -133,6 +133,10 @@ def load_findpairs(path: str = None):
     lib.fasted_find_epsilon_volumetric.restype = c.c_int
     lib.fasted_find_epsilon_volumetric.argtypes = [c.c_double, c.c_double, c.POINTER(c.c_double), c.POINTER(c.c_double),
                                                    c.POINTER(c.c_int)]
+    lib.fasted_set_download_pairs.restype = None
+    lib.fasted_set_download_pairs.argtypes = [c.c_int]
+    lib.fasted_last_pairs_device.restype = c.c_void_p
+    lib.fasted_last_pairs_device.argtypes = [c.POINTER(c.c_ulonglong)]
     lib.fasted_count_pairs_sampled.restype = c.c_int
     lib.fasted_count_pairs_sampled.argtypes = [c.c_double, c.c_int, c.POINTER(c.c_ulonglong), c.POINTER(c.c_int),
                                                c.POINTER(c.c_double)]
@@ -266,6 +270,18 @@ def pair_distances_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_
     lib = load_findpairs()
     _check(lib, lib.fasted_pair_distances_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates,
                                                  ld_candidates, d, pairs_ptr, count, distances_ptr, stream))
+
+
+def set_download_pairs(enabled):
+    """False: runs that do not save leave their pairs on the device (the reference always downloads them)."""
+    load_findpairs().fasted_set_download_pairs(1 if enabled else 0)
+
+
+def last_pairs_device():
+    """(device pointer, count) of the sorted pairs the last runFrom... / reRun stored; owned by the library."""
+    stored = ctypes.c_ulonglong()
+    ptr = load_findpairs().fasted_last_pairs_device(ctypes.byref(stored))
+    return ptr, stored.value
 
 
 def find_epsilon(target_selectivity, initial_epsilon=0.0):

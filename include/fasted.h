@@ -252,6 +252,14 @@ void fasted_set_output_dir(const char* dir);
  * source/pair.cuh:51-54. */
 void fasted_set_save_distances(int enabled);
 
+/* The reference copies the whole pair list to the host after every run, saved or not
+ * (source/findPairs.cuh:711-713: 16 GB per reRun at 2M x 384 with 1000 neighbours).  With a zero argument (or
+ * $FASTED_DOWNLOAD_PAIRS=0) a run that does not save leaves the pairs on the device; Results is unchanged.
+ * fasted_last_pairs_device: the sorted pairs of the last runFrom... / reRun in device memory (*stored of them),
+ * owned by the library, valid until the next run or releaseResources(). */
+void fasted_set_download_pairs(int enabled);
+const FastedPair* fasted_last_pairs_device(unsigned long long* stored);
+
 const char* fasted_last_error(void);
 const char* fasted_version(void);
 

@@ -1,5 +1,6 @@
 """GPU tests of the drop-in boundary: the reference's entry points, the `.pairs` text output and the
 command-line driver, checked against the CPU checker."""
+import ctypes
 import os
 import re
 import subprocess
@@ -117,6 +118,37 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     truth = oracle.self_join_f64(bits, eps, n=n)
     assert abs(int(found) - len(truth)) <= max(4, len(truth) // 500)
     lib.releaseResources()
+
+
+def test_pairs_can_stay_on_the_device(lib):
+    """With the download switched off a run that does not save reports the same Results and leaves the sorted pairs
+    in the library's device buffer, where fasted_last_pairs_device finds them; a saving run still writes its file."""
+    import torch
+
+    import fasted_amd
+
+    n, d = 3000, 64
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    bits, _, _, _ = fasted_amd.resident_points()
+    eps = datasets.epsilon_for_neighbours(bits[:n, :d].copy(), 12)
+    want, found = fasted_amd.self_join(bits[:n, :d].copy(), eps)
+    r_down = lib.reRun(eps, False)
+    fasted_amd.set_download_pairs(False)
+    try:
+        r = lib.reRun(eps, False)
+        assert (r.pairsFound, r.pairsStored) == (r_down.pairsFound, r_down.pairsStored) == (found, found)
+        ptr, stored = fasted_amd.last_pairs_device()
+        assert stored == found and ptr
+        out = torch.empty((stored, 2), dtype=torch.int32, device="cuda")
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        assert hip.hipMemcpy(out.data_ptr(), ptr, stored * 8, 3) == 0  # device to device
+        assert np.array_equal(out.cpu().numpy(), want)
+    finally:
+        fasted_amd.set_download_pairs(True)
+    lib.releaseResources()
+    ptr, stored = fasted_amd.last_pairs_device()
+    assert stored == 0
 
 
 def test_native_volumetric_epsilon_search(lib):
