@@ -42,7 +42,7 @@ constexpr int kOperandBytes = kTile * kRowBytes;    // 32 KiB per operand per st
 constexpr int kStageBytes = 2 * kOperandBytes;      // queries then candidates: 64 KiB
 constexpr int kLdsSums = 2 * kStageBytes;           // two buffers of s_q[256] then s_c[256] (current / next tile)
 constexpr int kSumsBytes = 2 * kTile * 4;
-constexpr int kLdsNext = kLdsSums + 2 * kSumsBytes; // next tile of this workgroup: (row, col) as two u32
+constexpr int kLdsNext = kLdsSums + 2 * kSumsBytes; // the next two tiles of this workgroup: two slots of (row, col) as u32
 constexpr int kLdsStage = kLdsNext + 16;            // staged pairs: one private region per wave
 constexpr int kWaveStagePairs = 384;                // 3 KiB of 8-byte records per wave
 constexpr int kLdsBytes = kLdsStage + 8 * kWaveStagePairs * 8;
@@ -239,7 +239,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 // sub-tile is 64 x 64, 4 x 4 blocks), so that twice as many workgroups find work.  The transfers stay as they
 // are -- 256 query rows from the tile's first row on are staged, the lower half unused -- which costs nothing
 // that matters at such sizes and keeps one set of addresses.
-template <bool kEpilogue, bool kTall, int kTileRows>
+// kOneSlab: D <= 64, a tile is one slab.  No barrier inside such a tile could publish the next tile's coordinates, so
+// the mailbox that carries them runs one tile further ahead there (two slots).
+template <bool kEpilogue, bool kTall, int kTileRows, bool kOneSlab>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     static_assert(kTileRows == 256 || kTileRows == 128, "tile rows");
     constexpr int kWaveRows = kTileRows / 2;    // rows of a wave's output sub-tile (2 x 4 waves)
@@ -265,7 +267,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     // LDS byte address of lds[0], for the LDS instructions written out by hand below
     const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // next tile: [0] row, [1] col
+    unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // two slots of [0] row, [1] col
     const int2* const sStage = reinterpret_cast<const int2*>(lds + kLdsStage) + wave * kWaveStagePairs;  // this wave's region
 
     // set by the kernel that formed the per-point halves: some point has a non-finite squared norm
@@ -391,7 +393,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
     // ---- first tile
     if (wave == 0 && lane_now() == 0) {
-        unsigned r, c;
+        unsigned r, c, r1 = kNoTile, c1 = 0u;
         if (p.direct) {
             // A matrix of no more tiles than workgroups: one tile each, by workgroup number.  Through the queues,
             // every workgroup would reserve a second tile while it starts its first (the reservation runs one
@@ -401,15 +403,20 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             if (p.symmetric && c < r) r = kNoTile;
         } else {
             find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r, &c);
+            if (kOneSlab && r != kNoTile) find_tile(atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull), &r1, &c1);
         }
+        // Single-slab tiles use two mailbox slots: during tile t, slot (t + 1) % 2 names tile t + 1 (written during
+        // tile t - 1 and published by the barrier at the top of tile t) and thread 0 writes tile t + 2 into slot
+        // t % 2.  With more slabs, slot 0 is written at the top of a tile and published by its first slab's barrier.
         sNext[0] = r;
         sNext[1] = c;
+        sNext[2] = r1;
+        sNext[3] = c1;
     }
     __syncthreads();
     unsigned tr = __builtin_amdgcn_readfirstlane(sNext[0]);
     unsigned tc = __builtin_amdgcn_readfirstlane(sNext[1]);
     if (tr == kNoTile) return;
-    __syncthreads();  // everybody has read sNext before thread 0 writes the second tile there
 
     unsigned offA[4], offB[4];
     tile_offsets((int)tr * kTileRows, (int)tc * kTile, offA, offB, true);
@@ -417,12 +424,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     const char* gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(tc) * kTile * p.ldC16);
     static_for<0, 8>([&](auto jc) { issue_load(jc, gA, gB, offA, offB, 0); });
     if (kNoTransfers) {
-        const int second = p.nSlabs > 1 ? kRowBytes : 0;
+        const int second = kOneSlab ? 0 : kRowBytes;
         static_for<0, 8>([&](auto jc) { issue_load(jc, gA + second, gB + second, offA, offB, 1); });
         filling = false;
     }
     issue_sums((int)tr * kTileRows, (int)tc * kTile, 0);
-    unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the current one
+    unsigned long long popped = 0;  // thread 0: the home queue position reserved for the tile after the next one to be decoded
     if (wave == 0 && lane_now() == 0 && !p.direct) popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
 
     int stage = 0;  // LDS stage that holds slab 0 of the current tile
@@ -441,8 +448,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                 find_tile(popped, &r, &c);
                 popped = atomicAdd(&p.counters[kQueueBase + home * kQueueStride], 1ull);
             }
-            sNext[0] = r;
-            sNext[1] = c;
+            const int slot = kOneSlab ? 2 * sumsBuf : 0;  // (sumsBuf is the tile count's parity)
+            sNext[slot] = r;
+            sNext[slot + 1] = c;
         }
 
         // The accumulators start at h_q + h_c, h = eps^2/4 - s/2 per point (see the epilogue): the tile's
@@ -594,7 +602,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 
         constexpr std::integral_constant<bool, true> kFirstSlab{};
         constexpr std::integral_constant<bool, false> kLaterSlab{};
-        if (p.nSlabs > 1) {
+        if (!kOneSlab && p.nSlabs > 1) {  // (the run-time test is always true here; the register allocator does better with it)
             slab_step(kFirstSlab, stage, true, gA + kRowBytes, gB + kRowBytes, offA, offB);
             stage ^= 1;
             transfers_landed_barrier();
@@ -604,13 +612,13 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             stage ^= 1;
             transfers_landed_barrier();
         }
-        if (p.nSlabs == 1) transfers_landed_barrier();  // with a single slab no barrier has published sNext yet
 
         // The tile after this one: its first slab and its squared norms travel during this tile's last
         // slab and epilogue.  The current tile's offsets are not needed any more, so the next tile's
         // take their registers.
-        const unsigned ntr = __builtin_amdgcn_readfirstlane(sNext[0]);
-        const unsigned ntc = __builtin_amdgcn_readfirstlane(sNext[1]);
+        const int slot = kOneSlab ? 2 * (sumsBuf ^ 1) : 0;
+        const unsigned ntr = __builtin_amdgcn_readfirstlane(sNext[slot]);
+        const unsigned ntc = __builtin_amdgcn_readfirstlane(sNext[slot + 1]);
         const bool more = ntr != kNoTile;
         if (more) {
             tile_offsets((int)ntr * kTileRows, (int)ntc * kTile, offA, offB, false);
@@ -618,7 +626,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             gB = reinterpret_cast<const char*>(p.ptsC + (long long)panel_of(ntc) * kTile * p.ldC16);
             issue_sums((int)ntr * kTileRows, (int)ntc * kTile, sumsBuf ^ 1);
         }
-        if (p.nSlabs == 1) {  // a single slab: all rows are set before it
+        if (kOneSlab || p.nSlabs == 1) {  // a single slab: all rows are set before it
 #pragma unroll
             for (int fi = 1; fi < kFragRows; ++fi) init_row(fi);
         }
@@ -934,16 +942,25 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
     if (grid == 0) grid = 1;
     const bool tall = tall_order(l.nQ, tileRows);
     const dim3 g(grid), b(kThreads);
-    const int variant = (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
+    const bool oneSlab = p.nSlabs == 1;
+    const int variant = (oneSlab ? 8 : 0) | (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
     switch (variant) {
-        case 7: join_kernel<true, true, 128><<<g, b, 0, stream>>>(p); break;
-        case 6: join_kernel<true, true, 256><<<g, b, 0, stream>>>(p); break;
-        case 5: join_kernel<true, false, 128><<<g, b, 0, stream>>>(p); break;
-        case 4: join_kernel<true, false, 256><<<g, b, 0, stream>>>(p); break;
-        case 3: join_kernel<false, true, 128><<<g, b, 0, stream>>>(p); break;
-        case 2: join_kernel<false, true, 256><<<g, b, 0, stream>>>(p); break;
-        case 1: join_kernel<false, false, 128><<<g, b, 0, stream>>>(p); break;
-        default: join_kernel<false, false, 256><<<g, b, 0, stream>>>(p); break;
+        case 15: join_kernel<true, true, 128, true><<<g, b, 0, stream>>>(p); break;
+        case 14: join_kernel<true, true, 256, true><<<g, b, 0, stream>>>(p); break;
+        case 13: join_kernel<true, false, 128, true><<<g, b, 0, stream>>>(p); break;
+        case 12: join_kernel<true, false, 256, true><<<g, b, 0, stream>>>(p); break;
+        case 11: join_kernel<false, true, 128, true><<<g, b, 0, stream>>>(p); break;
+        case 10: join_kernel<false, true, 256, true><<<g, b, 0, stream>>>(p); break;
+        case 9: join_kernel<false, false, 128, true><<<g, b, 0, stream>>>(p); break;
+        case 8: join_kernel<false, false, 256, true><<<g, b, 0, stream>>>(p); break;
+        case 7: join_kernel<true, true, 128, false><<<g, b, 0, stream>>>(p); break;
+        case 6: join_kernel<true, true, 256, false><<<g, b, 0, stream>>>(p); break;
+        case 5: join_kernel<true, false, 128, false><<<g, b, 0, stream>>>(p); break;
+        case 4: join_kernel<true, false, 256, false><<<g, b, 0, stream>>>(p); break;
+        case 3: join_kernel<false, true, 128, false><<<g, b, 0, stream>>>(p); break;
+        case 2: join_kernel<false, true, 256, false><<<g, b, 0, stream>>>(p); break;
+        case 1: join_kernel<false, false, 128, false><<<g, b, 0, stream>>>(p); break;
+        default: join_kernel<false, false, 256, false><<<g, b, 0, stream>>>(p); break;
     }
     return hipGetLastError();
 }
