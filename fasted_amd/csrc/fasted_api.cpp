@@ -648,6 +648,7 @@ Results find_pairs_resident(double epsilon, bool savePairs, bool skipUpload, con
     }
     HIP_CHECK(hipDeviceSynchronize());
 
+    g_lastStored = 0;  // the buffer may move or be overwritten from here on
     const unsigned long long maxPairs = std::min(ensure_pair_buffer(tb.n), g_pairWs.capPairs);
     g_pairWs.ensure_host();
     void* const dPairs = g_pairWs.dPairs;
