@@ -14,6 +14,10 @@
 //                        reservation per workgroup flush instead of two atomics per pair
 //                        (source/pair.cuh:123-133).  The first slab and the squared norms of the
 //                        next tile travel during the last slab and the epilogue of the current one.
+//                        Variants of the same code: tiles of 128 query rows and one workgroup per tile
+//                        without the queues for matrices of few tiles (the reference runs smaller tiles
+//                        on more blocks, source/findPairs.cuh:55-63,656), and a mailbox that runs one tile
+//                        further ahead for tiles of a single slab (D <= 64).
 //
 // Data layout: points are row-major FP16, one point per row, row stride `ld` halves.  Both
 // MFMA operands are "row = point, 8 consecutive k per lane", so the query tile and the
