@@ -63,9 +63,16 @@ struct Workspace {
     float* sums = nullptr;
     float* halves = nullptr;
     size_t cap = 0;
+    // kept between calls, so that a small join does not pay for them every time: the three timing events and a
+    // pinned word the pair counter is copied into behind the join kernel (one wait for kernels and count)
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    unsigned long long* hostCount = nullptr;
 
     void ensure(size_t n) {
         if (!counters) HIP_CHECK(hipMalloc(&counters, fasted::counter_words() * sizeof(unsigned long long)));
+        if (!hostCount) HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocDefault));
+        for (auto& e : ev)
+            if (!e) HIP_CHECK(hipEventCreate(&e));
         if (n > cap) {
             if (sums) HIP_CHECK(hipFree(sums));
             if (halves) HIP_CHECK(hipFree(halves));
@@ -80,8 +87,14 @@ struct Workspace {
         if (counters) (void)hipFree(counters);
         if (sums) (void)hipFree(sums);
         if (halves) (void)hipFree(halves);
+        if (hostCount) (void)hipHostFree(hostCount);
+        for (auto& e : ev) {
+            if (e) (void)hipEventDestroy(e);
+            e = nullptr;
+        }
         counters = nullptr;
         sums = halves = nullptr;
+        hostCount = nullptr;
         cap = 0;
     }
 } g_ws;
@@ -184,7 +197,8 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     validate_shape(c.n, d, c.ld);
     if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
     const int dPad = round_up(d, fasted::kSlabK);
-    EventTimer t(fixed ? fixed->ev : nullptr);
+    if (!fixed) g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
+    EventTimer t(fixed ? fixed->ev : g_ws.ev);
     unsigned long long* counters = nullptr;
     float* wsSums = nullptr;
     float* wsHalves = nullptr;
@@ -193,7 +207,6 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
         wsSums = fixed->sums;
         wsHalves = fixed->halves;
     } else {
-        g_ws.ensure((size_t)q.n + (selfJoin ? 0 : (size_t)c.n));
         counters = g_ws.counters;
         wsSums = g_ws.sums;
         wsHalves = g_ws.halves;
@@ -238,12 +251,18 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
     HIP_CHECK(fasted::launch_join(jl, stream));
     HIP_CHECK(hipEventRecord(t.ev[2], stream));
-    HIP_CHECK(hipStreamSynchronize(stream));
-
     // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
     // counted only (source/pair.cuh:123-133), so stored = min(found, capacity)
     unsigned long long cnt[4] = {0, 0, 0, 0};
-    HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    if (fixed) {
+        HIP_CHECK(hipStreamSynchronize(stream));
+        HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    } else {
+        // the count travels behind the join kernel into pinned memory: one wait for both
+        HIP_CHECK(hipMemcpyAsync(g_ws.hostCount, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        cnt[0] = *g_ws.hostCount;
+    }
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);
     if (jl.symmetric) {
