@@ -314,12 +314,14 @@ def find_epsilon_sampled(target_selectivity, sample_rows=16384, initial_epsilon=
 
 
 def join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates, d, epsilon, pairs_ptr,
-                cap, flags=FASTED_SORT_PAIRS, stream=None):
-    """Join of two different point sets on raw device pointers; returns FastedJoinStats."""
+                cap, flags=FASTED_SORT_PAIRS, stream=None, sums_queries_ptr=None, sums_candidates_ptr=None):
+    """Join of two different point sets on raw device pointers; returns FastedJoinStats.  The two optional
+    squared-norm buffers are filled by the call, or read by it with FASTED_SKIP_SUMS."""
     lib = load_findpairs()
     st = FastedJoinStats()
     _check(lib, lib.fasted_join_device(queries_ptr, n_queries, ld_queries, candidates_ptr, n_candidates, ld_candidates,
-                                       d, float(epsilon), None, None, pairs_ptr, cap, flags, stream, ctypes.byref(st)))
+                                       d, float(epsilon), sums_queries_ptr, sums_candidates_ptr, pairs_ptr, cap, flags,
+                                       stream, ctypes.byref(st)))
     return st
 
 
