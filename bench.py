@@ -9,8 +9,9 @@ resident in HBM before the timed region starts.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3]
 
 prints ONE JSON line: metric = self-join TFLOPS (2*N^2*D / time), plus `roofline`
-(the join kernel against the dense FP16 MFMA peak) and `cpu_baseline` (the FP64 brute-force
-checker timed on this box's host cores on a bounded sample of the same workload).
+(the join kernel against the dense FP16 MFMA peak) and `cpu_baseline` (a blocked FP64 / FP32 brute-force
+join timed on this box's host cores: in full for the small workloads, else on 1024 seeded query rows
+against all points).
 """
 import argparse
 import json
@@ -125,35 +126,70 @@ def parity_sample(torch, pts, eps, pairs, stored, rows=1024, seed=7, band=1e-3):
             "outside_band": outside, "max_rel_distance_error": worst, "band": band}
 
 
-def cpu_baseline(torch, pts, eps, budget_s=15.0):
-    """FP64 brute-force join (the CPU checker) on a bounded sample: Q query rows against the
-    first Nc points of the same dataset, on this box's host cores."""
+def cpu_baseline(torch, pts, eps, full_limit=2.0e5, sample_rows=1024, budget_s=100.0, seed=99):
+    """Blocked brute-force join on this box's host cores (oracle/blocked_join.c: GEMM form, cache blocked,
+    OpenMP), FP64 and FP32, same pair definition as the GPU join.  Small workloads (N <= full_limit) run in
+    full; the others join `sample_rows` seeded query rows with ALL N candidates and the time is extrapolated
+    linearly (x N / rows), labelled as such.  Candidates are streamed from the device in chunks, every chunk
+    is joined three times per precision, the per-pass totals give the median of three.  Only time spent inside
+    the join routine counts (the dataset is "already in memory")."""
     import numpy as np
 
     import oracle
 
     n, d = pts.shape
-    nc = int(min(n, max(1024, (1 << 27) // d)))
-    host = pts[:nc].cpu().numpy().view(np.uint16)
-    cores = min(oracle.num_threads(), 16)
-    os.environ["OMP_NUM_THREADS"] = str(cores)
+    threads = oracle.num_threads()
+    full = n <= full_limit
+    if full:
+        rows = torch.arange(n, device="cuda")
+    else:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        rows = torch.sort(torch.randperm(n, generator=g, device="cuda")[:sample_rows]).values
+    q = pts[rows].cpu().numpy().view(np.uint16)
+    nq = q.shape[0]
+    chunk = int(max(1024, min(n, (1 << 27) // d)))
+    chunks = [(c0, min(n, c0 + chunk)) for c0 in range(0, n, chunk)]
+    passes = {64: [0.0, 0.0, 0.0], 32: [0.0, 0.0, 0.0]}
+    found = {64: [0, 0, 0], 32: [0, 0, 0]}
+    repeats = 3
+    for i, (c0, c1) in enumerate(chunks):
+        c = pts[c0:c1].cpu().numpy().view(np.uint16)
+        for precision in (64, 32):
+            for r in range(repeats):
+                _, f, secs = oracle.blocked_join(q, c, eps, precision, want_pairs=False)
+                passes[precision][r] += secs
+                found[precision][r] += f
+        if i == 0 and repeats == 3:
+            # one pass only when three would not fit the budget (said in `median_of`)
+            projected = (passes[64][0] + passes[32][0]) * len(chunks) * 3
+            if projected > budget_s:
+                repeats = 1
+        del c
 
-    def run(q):
-        t0 = time.perf_counter()
-        pairs = oracle.self_join_f64(host, eps, n=nc, rows=(0, q))
-        return time.perf_counter() - t0, len(pairs)
+    def rate(precision):
+        t = sorted(passes[precision][:repeats])[repeats // 2]
+        return {"tflops": 2.0 * nq * n * d / t / 1e12, "seconds": t, "pairs_found": int(found[precision][0]),
+                "pairs_per_s": found[precision][0] / t, "extrapolated_full_seconds": t * n / nq}
 
-    q = min(nc, max(cores * 4, 64))
-    t, _ = run(q)
-    q2 = int(min(nc, max(q, q * budget_s / max(t, 1e-3))))
-    if q2 > q:
-        t, _ = run(q2)
-        q = q2
-    tflops = 2.0 * q * nc * d / t / 1e12
+    fp64, fp32 = rate(64), rate(32)
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    what = "all" if full else f"{nq} seeded"
     return {
-        "value": tflops, "unit": "TFLOPS", "cores": cores, "kind": "port",
-        "sample": f"{q} query rows x first {nc} points x D={d}, FP64, {t:.2f} s "
-                  f"(full-size extrapolation: {2.0 * n * n * d / (tflops * 1e12):.0f} s)",
+        "value": fp32["tflops"], "unit": "TFLOPS", "cores": threads, "kind": "port", "precision_of_value": "fp32",
+        "sample": f"{what} query rows x all {n} candidates x D={d} ({'full join' if full else 'time x N/rows is an extrapolation'}), "
+                  f"blocked GEMM-form join, {oracle.blocked_join_vector_bits()}-bit vectors",
+        "fp64": fp64, "fp32": fp32, "threads": threads, "nproc": os.cpu_count(),
+        "affinity": len(os.sched_getaffinity(0)), "cpu_model": model, "median_of": repeats,
+        "query_rows": nq, "full": bool(full),
     }
 
 
@@ -244,6 +280,8 @@ def main():
     ap.add_argument("--no-epilogue", action="store_true", help="measurement: contraction only")
     ap.add_argument("--no-symmetric-option", action="store_true",
                     help="skip the extra launch that measures the opt-in FASTED_SYMMETRIC mode")
+    ap.add_argument("--allow-ablation", action="store_true",
+                    help="measurement: accept a library built with parts of the join kernel compiled out (FASTED_LIBRARY)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 1 GiB read + 1 GiB write elementwise kernel (to scale FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -260,7 +298,13 @@ def main():
     if not torch.cuda.is_available():
         print("no GPU visible: the join has no CPU fallback", file=sys.stderr)
         sys.exit(1)
-    fasted_amd.load_findpairs()
+    lib = fasted_amd.load_findpairs()
+    version = lib.fasted_version().decode()
+    ablation = "ABLATION" in version
+    if ablation and not (args.no_epilogue or args.allow_ablation):
+        print(f"refusing to benchmark a measurement build as the product: {version} (pass --allow-ablation to time "
+              "it; its line then says what it is and carries no parity claim)", file=sys.stderr)
+        sys.exit(4)
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
@@ -315,7 +359,8 @@ def main():
                    "mean_neighbours": (st.pairsFound - n) / n, "pairs_per_s": st.pairsFound / (ms_per_step / 1000.0),
                    "pct_of_fp16_peak": 100.0 * tflops / PEAK_FP16_TFLOPS, "tiles": int(st.tiles),
                    "sum_squared_ms": sums_ms, "join_kernel_ms": join_ms, "epilogue": not args.no_epilogue,
-                   "accumulate": "f32", "peak_used_tflops": PEAK_FP16_TFLOPS, "clocks": clocks.summary()},
+                   "accumulate": "f32", "library": version,
+                   "library_path": fp.library_path(), "peak_used_tflops": PEAK_FP16_TFLOPS, "clocks": clocks.summary()},
         "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
                      "traffic": traffic, "traffic_detail": traffic_detail},
@@ -324,7 +369,11 @@ def main():
     # relative 1e-3 band around epsilon, a pair buffer that overflowed so that nothing could be checked, a
     # symmetric-mode count that differs) says so and the process exits non-zero.
     problems = []
-    if not args.no_epilogue:
+    if ablation:
+        args.no_symmetric_option = True
+        out["config"]["parity_ok"] = None
+        out["config"]["note"] = "measurement build: results are wrong by construction, no parity claim"
+    if not args.no_epilogue and not ablation:
         if st.pairsStored == st.pairsFound:
             out["config"]["parity_vs_fp64"] = parity_sample(torch, pts, eps, pairs, int(st.pairsStored))
             if out["config"]["parity_vs_fp64"]["outside_band"] > 0:
@@ -346,7 +395,8 @@ def main():
             problems.append("symmetric mode found a different number of pairs")
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, pts, eps)
-    if not args.no_epilogue:
+        out["cpu_baseline"]["gpu_over_cpu"] = tflops / out["cpu_baseline"]["value"]
+    if not args.no_epilogue and not ablation:
         out["config"]["parity_ok"] = not problems
         if problems:
             out["config"]["parity_problems"] = problems

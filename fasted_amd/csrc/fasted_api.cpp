@@ -67,10 +67,26 @@ struct Workspace {
     // pinned word the pair counter is copied into behind the join kernel (one wait for kernels and count)
     hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
     unsigned long long* hostCount = nullptr;
+    unsigned long long* hostCountDev = nullptr;  // the same words as the device addresses them
+    double clockRate = 0.0;
+
+    // ticks per millisecond of the clock the kernels read (a constant-rate counter, independent of the shader clock)
+    double clockKHz() {
+        if (clockRate == 0.0) {
+            int dev = 0, khz = 0;
+            HIP_CHECK(hipGetDevice(&dev));
+            HIP_CHECK(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+            clockRate = khz > 0 ? (double)khz : 100000.0;
+        }
+        return clockRate;
+    }
 
     void ensure(size_t n) {
         if (!counters) HIP_CHECK(hipMalloc(&counters, fasted::counter_words() * sizeof(unsigned long long)));
-        if (!hostCount) HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocDefault));
+        if (!hostCount) {
+            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocDefault));
+            HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&hostCountDev), hostCount, 0));
+        }
         for (auto& e : ev)
             if (!e) HIP_CHECK(hipEventCreate(&e));
         if (n > cap) {
@@ -94,7 +110,7 @@ struct Workspace {
         }
         counters = nullptr;
         sums = halves = nullptr;
-        hostCount = nullptr;
+        hostCount = hostCountDev = nullptr;
         cap = 0;
     }
 } g_ws;
@@ -140,6 +156,10 @@ struct JoinScratch {
     hipEvent_t* ev;  // three events
 };
 
+// Joins are numbered: the norm kernels of a join write its number into the non-finite flag of the counter
+// block, the join kernel compares with it, and so the flag never has to be cleared between joins.
+unsigned long long g_epoch = 0;
+
 fasted::SortBuffers g_sortWs;  // device buffers of the row-major sort, kept between calls
 
 // Three events around the two timed stages; created for the call, or borrowed from the caller.
@@ -168,6 +188,12 @@ struct EventTimer {
     }
 };
 
+// A NaN epsilon compares false with every distance in the reference (source/warpMma.cuh:257: no pairs at all);
+// here the accumulator start values are formed from epsilon, so it is refused before any launch.
+void validate_epsilon(double epsilon) {
+    if (std::isnan(epsilon)) throw std::invalid_argument("epsilon is NaN");
+}
+
 void validate_shape(long long n, int d, long long ld) {
     if (n < 1) throw std::invalid_argument("number of points must be at least 1");
     if (n > (long long)INT_MAX - 2 * fasted::kTile) throw std::invalid_argument("number of points exceeds int range");
@@ -193,6 +219,7 @@ struct PointSet {
 void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon, void* dPairs,
                     unsigned long long cap, unsigned flags, hipStream_t stream, FastedJoinStats* stats,
                     const JoinScratch* fixed = nullptr, bool sortMayFail = false, int forcedStride = 0) {
+    validate_epsilon(epsilon);
     validate_shape(q.n, d, q.ld);
     validate_shape(c.n, d, c.ld);
     if (cap > 0 && !dPairs) throw std::invalid_argument("pair buffer is null");
@@ -220,17 +247,26 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     const float eps2 = static_cast<float>(epsilon * epsilon);  // product in double, then narrowed (findPairs.cuh:678)
 
     // squared norms and, from them, each point's accumulator start value eps^2/4 - s/2
-    HIP_CHECK(hipEventRecord(t.ev[0], stream));
-    HIP_CHECK(fasted::launch_reset_counters(counters, false, stream));
+    // (the first of these launches also clears the pair counter and the queue heads)
+    const unsigned long long epoch = ++g_epoch;
+    // Timing.  Three event records cost a call about 10 us, a third of a join of a few thousand points, so a
+    // join of at most two tiles per compute unit is timed by the kernels themselves instead: the first norm
+    // kernel and the join kernel note the device's constant-rate clock when they start, and so does the
+    // one-thread kernel behind the join that hands the pair count to the host.  Larger joins, and the entry
+    // that owns no pinned memory, are timed with events on the stream as the reference is
+    // (source/findPairs.cuh:625-639,695-697,728-736).
+    const bool stamped = !fixed && fasted::tile_count(q.n, c.n) <= 512;
+    const bool events = !stamped && stats != nullptr;
+    if (events) HIP_CHECK(hipEventRecord(t.ev[0], stream));
     if (!(flags & FASTED_SKIP_SUMS)) {
-        HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, halfQ, eps2, counters, stream));
+        HIP_CHECK(fasted::launch_sum_squared(q.ptr, q.ld, (int)q.n, dPad, sumsQ, halfQ, eps2, counters, stream, epoch, true));
         if (!selfJoin)
-            HIP_CHECK(fasted::launch_sum_squared(c.ptr, c.ld, (int)c.n, dPad, sumsC, halfC, eps2, counters, stream));
+            HIP_CHECK(fasted::launch_sum_squared(c.ptr, c.ld, (int)c.n, dPad, sumsC, halfC, eps2, counters, stream, epoch));
     } else {
-        HIP_CHECK(fasted::launch_halves(sumsQ, (int)q.n, eps2, halfQ, counters, stream));
-        if (!selfJoin) HIP_CHECK(fasted::launch_halves(sumsC, (int)c.n, eps2, halfC, counters, stream));
+        HIP_CHECK(fasted::launch_halves(sumsQ, (int)q.n, eps2, halfQ, counters, stream, epoch, true));
+        if (!selfJoin) HIP_CHECK(fasted::launch_halves(sumsC, (int)c.n, eps2, halfC, counters, stream, epoch));
     }
-    HIP_CHECK(hipEventRecord(t.ev[1], stream));
+    if (events) HIP_CHECK(hipEventRecord(t.ev[1], stream));
 
     fasted::JoinLaunch jl;
     jl.queries = q.ptr;
@@ -246,11 +282,12 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.halfQ = halfQ;
     jl.halfC = halfC;
     jl.counters = counters;
+    jl.epoch = epoch;
     jl.pairs = dPairs;
     jl.cap = cap;
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
     HIP_CHECK(fasted::launch_join(jl, stream));
-    HIP_CHECK(hipEventRecord(t.ev[2], stream));
+    if (events) HIP_CHECK(hipEventRecord(t.ev[2], stream));
     // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
     // counted only (source/pair.cuh:123-133), so stored = min(found, capacity)
     unsigned long long cnt[4] = {0, 0, 0, 0};
@@ -258,10 +295,11 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
         HIP_CHECK(hipStreamSynchronize(stream));
         HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
     } else {
-        // the count travels behind the join kernel into pinned memory: one wait for both
-        HIP_CHECK(hipMemcpyAsync(g_ws.hostCount, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost, stream));
+        // the count (and the kernels' clock readings) travel behind the join kernel into pinned memory, written
+        // by a one-thread kernel: one wait for kernels and count
+        HIP_CHECK(fasted::launch_publish_count(counters, g_ws.hostCountDev, stream));
         HIP_CHECK(hipStreamSynchronize(stream));
-        cnt[0] = *g_ws.hostCount;
+        cnt[0] = static_cast<volatile unsigned long long*>(g_ws.hostCount)[0];
     }
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);
@@ -281,8 +319,14 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
         sortMs = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
     }
     if (stats) {
-        stats->sumSquaredMs = t.ms(0, 1);
-        stats->joinMs = t.ms(1, 2);
+        if (stamped) {
+            const volatile unsigned long long* const w = g_ws.hostCount;  // [1] norms start, [2] join start, [3] join over
+            stats->sumSquaredMs = (float)((double)(w[2] - w[1]) / g_ws.clockKHz());
+            stats->joinMs = (float)((double)(w[3] - w[2]) / g_ws.clockKHz());
+        } else {
+            stats->sumSquaredMs = t.ms(0, 1);
+            stats->joinMs = t.ms(1, 2);
+        }
         stats->sortMs = sortMs;
         stats->paddedN = round_up(q.n, fasted::kTile);
         stats->paddedD = dPad;
@@ -333,6 +377,22 @@ void upload_rows(void* dst, size_t pitch, const void* src, size_t rowBytes, size
     HIP_CHECK(hipStreamSynchronize(stream));  // the staging buffers go away with this frame
 }
 
+// The largest pair count <= `want` whose records fit the free device memory together with what the sort of
+// that many records needs beside them (a second key buffer and the radix sort's storage), as Pairs::init
+// shrinks the reference's buffer to the free memory (source/pair.cuh:69-85).
+unsigned long long fit_pairs_with_sort(unsigned long long want) {
+    size_t freeB = 0, totalB = 0;
+    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
+    const size_t usable = freeB - freeB / 16;  // leave some room for the runtime
+    unsigned long long maxPairs = want;
+    for (int round = 0; round < 4; ++round) {
+        const size_t need = (size_t)maxPairs * sizeof(FastedPair) + fasted::sort_scratch_bytes(maxPairs);
+        if (need <= usable) break;
+        maxPairs = (unsigned long long)((double)maxPairs * (double)usable / (double)need * 0.98);
+    }
+    return maxPairs;
+}
+
 // Self-join of a host-resident dataset that is streamed through the device in blocks of `blockRows`
 // points: for every query block (held on the device) every candidate block is uploaded in turn, on a
 // copy stream, while the join of the block before it runs.  The pairs of one query block are appended
@@ -359,6 +419,7 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
     if (!points) throw std::invalid_argument("points pointer is null");
     if (cap > 0 && !out) throw std::invalid_argument("output buffer is null");
     if (blockRows < 1) throw std::invalid_argument("block size must be at least 1 point");
+    validate_epsilon(epsilon);
     const int dPad = round_up(d, fasted::kSlabK);
     validate_shape(n, d, dPad);
     // blocks start on tile boundaries, so a block join sees the same tiles as the whole join would
@@ -366,91 +427,133 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
     const long long blocks = (n + rows - 1) / rows;
     const size_t pitch = (size_t)dPad * 2, blockBytes = (size_t)rows * pitch;
 
+    // Three block buffers.  One holds the query block; the candidate blocks pass through the other two, and
+    // the order of the candidates is chosen so that nothing is uploaded twice in a row: the last candidate of
+    // query block i is block i + 1, whose buffer then becomes the query buffer, and the old query block is
+    // still resident as the first off-diagonal candidate of block i + 1.  Uploads run on a copy stream while
+    // joins run on the compute stream; events, not the host, order a buffer's upload behind the last join
+    // that read it and a join behind the upload of its candidates.
     DeviceBuffers dev;
     HIP_CHECK(hipStreamCreateWithFlags(&dev.compute, hipStreamNonBlocking));
     HIP_CHECK(hipStreamCreateWithFlags(&dev.copy, hipStreamNonBlocking));
-    void* qBlock = dev.alloc(blockBytes);
-    void* cBlock[2] = {dev.alloc(blockBytes), dev.alloc(blockBytes)};
-    // per-point accumulator start values of the query block and of the two candidate buffers
-    float* qSums = static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)));
-    float* cSums[2] = {static_cast<float*>(dev.alloc((size_t)rows * sizeof(float))),
-                       static_cast<float*>(dev.alloc((size_t)rows * sizeof(float)))};
+    struct BlockBuffer {
+        void* rows = nullptr;
+        long long block = -1;           // which block of the dataset it holds
+        hipEvent_t uploaded = nullptr;  // recorded on the copy stream behind the upload
+        hipEvent_t released = nullptr;  // recorded on the compute stream behind the last join that read it
+    } buf[3];
+    struct Events {
+        BlockBuffer* b;
+        ~Events() {
+            for (int i = 0; i < 3; ++i) {
+                if (b[i].uploaded) (void)hipEventDestroy(b[i].uploaded);
+                if (b[i].released) (void)hipEventDestroy(b[i].released);
+            }
+        }
+    } eventGuard{buf};
+    for (auto& b : buf) {
+        b.rows = dev.alloc(blockBytes);
+        HIP_CHECK(hipEventCreateWithFlags(&b.uploaded, hipEventDisableTiming));
+        HIP_CHECK(hipEventCreateWithFlags(&b.released, hipEventDisableTiming));
+    }
+    // accumulator start values eps^2/4 - s/2 of every point of the dataset: formed when a block is uploaded
+    // for the first time (all of them during the first query block), read again for every later query block
+    float* const halves = static_cast<float*>(dev.alloc((size_t)blocks * rows * sizeof(float)));
+    std::vector<char> haveHalves((size_t)blocks, 0);
+    // where the pairs of the joins of one query block begin: mark[k] = pair counter before its k-th join
+    unsigned long long* const marks =
+        static_cast<unsigned long long*>(dev.alloc((size_t)(blocks + 1) * sizeof(unsigned long long)));
     // pair buffer of one query block: rows*256 records as the reference sizes its buffer per point
-    // (source/findPairs.cuh:644-647), shrunk to half of what is free (the sort needs as much again)
+    // (source/findPairs.cuh:644-647), shrunk to what is free together with the sort's own buffers
     unsigned long long devCap = std::min<unsigned long long>((unsigned long long)rows * 256ull, cap);
-    size_t freeB = 0, totalB = 0;
-    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
-    devCap = std::min<unsigned long long>(devCap, (unsigned long long)(freeB / 2) / sizeof(FastedPair));
+    devCap = fit_pairs_with_sort(devCap);
     void* dPairs = dev.alloc((size_t)devCap * sizeof(FastedPair));
     g_ws.ensure(1);
 
     auto block_rows = [&](long long b) { return std::min<long long>(rows, n - b * rows); };
-    auto upload = [&](void* dst, long long b, hipStream_t s) {
-        upload_rows(dst, pitch, points + (size_t)b * rows * d, (size_t)d * 2, (size_t)block_rows(b), s);
-    };
-    unsigned long long foundAll = 0, storedAll = 0;
     const float eps2 = static_cast<float>(epsilon * epsilon);
+    const unsigned long long epoch = ++g_epoch;  // one number for all block joins of this call
+    // Block b into buffer `into`, on the copy stream, once the joins that still read the buffer are through.
+    auto upload = [&](BlockBuffer& into, long long b) {
+        HIP_CHECK(hipStreamWaitEvent(dev.copy, into.released, 0));
+        upload_rows(into.rows, pitch, points + (size_t)b * rows * d, (size_t)d * 2, (size_t)block_rows(b), dev.copy);
+        HIP_CHECK(hipEventRecord(into.uploaded, dev.copy));
+        into.block = b;
+    };
+    // The compute stream waits for the upload of a buffer and forms the block's start values if they are new.
+    auto make_ready = [&](BlockBuffer& b) {
+        HIP_CHECK(hipStreamWaitEvent(dev.compute, b.uploaded, 0));
+        if (!haveHalves[(size_t)b.block]) {
+            HIP_CHECK(fasted::launch_sum_squared(b.rows, dPad, (int)block_rows(b.block), dPad, nullptr,
+                                                 halves + (size_t)b.block * rows, eps2, g_ws.counters, dev.compute, epoch));
+            haveHalves[(size_t)b.block] = 1;
+        }
+    };
+
+    unsigned long long foundAll = 0, storedAll = 0;
+    BlockBuffer* query = &buf[0];
+    BlockBuffer* spare[2] = {&buf[1], &buf[2]};
+    for (auto& b : buf) HIP_CHECK(hipEventRecord(b.released, dev.compute));
+    upload(*query, 0);
     for (long long i = 0; i < blocks; ++i) {
         const int nQ = (int)block_rows(i);
-        upload(qBlock, i, dev.compute);
+        make_ready(*query);
         HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, false, dev.compute));
-        HIP_CHECK(fasted::launch_sum_squared(qBlock, dPad, nQ, dPad, nullptr, qSums, eps2, g_ws.counters, dev.compute));
-        unsigned long long before = 0;  // pairs of this query block found so far
-        // candidate blocks other than block i itself pass through the two buffers in turn; `nextUp` is the
-        // block to upload next, cBlock[slot] the buffer the next such join reads
-        auto other_after = [&](long long b) { return (b + 1 == i) ? b + 2 : b + 1; };
-        long long nextUp = (i == 0) ? 1 : 0;
-        int slot = 0;
-        if (nextUp < blocks) {
-            upload(cBlock[0], nextUp, dev.copy);
-            nextUp = other_after(nextUp);
-        }
-        for (long long j = 0; j < blocks; ++j) {
-            const bool diagonal = (j == i);
-            const void* cand = qBlock;
-            const float* candSums = qSums;
-            int nC = nQ;
-            if (!diagonal) {
-                HIP_CHECK(hipStreamSynchronize(dev.copy));  // block j has arrived in cBlock[slot]
-                cand = cBlock[slot];
-                candSums = cSums[slot];
-                nC = (int)block_rows(j);
-                HIP_CHECK(fasted::launch_sum_squared(cand, dPad, nC, dPad, nullptr, cSums[slot], eps2, g_ws.counters,
-                                                     dev.compute));
-            }
+        HIP_CHECK(hipMemsetAsync(marks, 0, sizeof(unsigned long long), dev.compute));
+        // Candidates in this order: block i itself (the query buffer), then what the two spare buffers still
+        // hold from the query block before (block i - 1 in spare[0], some other block in spare[1]), then the
+        // rest, block i + 1 last.  Position p >= 1 of the order lives in spare[(p - 1) % 2]: the joins read
+        // the two buffers in turn, and a buffer receives position p behind join p - 2, which read it.
+        std::vector<long long> order{i};
+        const bool keep0 = i > 0 && spare[0]->block == i - 1;
+        if (keep0) order.push_back(i - 1);
+        const long long held = spare[1]->block;
+        const bool keep1 = keep0 && held >= 0 && held != i && held != i - 1 && held != i + 1;
+        if (keep1) order.push_back(held);
+        for (long long j = 0; j < blocks; ++j)
+            if (j != i && j != i + 1 && !(keep0 && j == i - 1) && !(keep1 && j == held)) order.push_back(j);
+        if (i + 1 < blocks) order.push_back(i + 1);
+        size_t next = 1 + (keep0 ? 1 : 0) + (keep1 ? 1 : 0);  // first position that has to be uploaded
+        for (size_t k = 0; k < order.size(); ++k) {
+            const long long j = order[k];
+            const bool diagonal = (k == 0);
+            BlockBuffer& cand = diagonal ? *query : *spare[(k - 1) % 2];
+            if (cand.block != j) throw std::logic_error("blocked join: a candidate block is not where it should be");
+            if (!diagonal) make_ready(cand);
             fasted::JoinLaunch jl;
-            jl.queries = qBlock;
-            jl.candidates = cand;
+            jl.queries = query->rows;
+            jl.candidates = cand.rows;
             jl.ldQ = jl.ldC = dPad;
             jl.nQ = nQ;
-            jl.nC = nC;
+            jl.nC = (int)block_rows(j);
             jl.selfJoin = diagonal;
             jl.symmetric = false;
             jl.dPad = dPad;
-            jl.halfQ = qSums;
-            jl.halfC = candSums;
+            jl.halfQ = halves + (size_t)i * rows;
+            jl.halfC = halves + (size_t)j * rows;
             jl.counters = g_ws.counters;
+            jl.epoch = epoch;
             jl.pairs = dPairs;
             jl.cap = devCap;
             jl.epilogue = true;
             HIP_CHECK(fasted::launch_reset_counters(g_ws.counters, /*keepFound=*/true, dev.compute));
             HIP_CHECK(fasted::launch_join(jl, dev.compute));
-            if (!diagonal) {
-                // the next candidate block travels while this join runs; the other buffer was last read
-                // by a join that has finished (its counter was read back)
-                slot ^= 1;
-                if (nextUp < blocks) {
-                    upload(cBlock[slot], nextUp, dev.copy);
-                    nextUp = other_after(nextUp);
-                }
+            // block-local indices -> indices of the whole dataset, for the pairs this join appended
+            HIP_CHECK(fasted::launch_offset_appended_pairs(dPairs, marks + k, g_ws.counters, devCap, (int)(i * rows),
+                                                           (int)(j * rows), dev.compute));
+            if (!diagonal) HIP_CHECK(hipEventRecord(cand.released, dev.compute));
+            // With join k queued, the host turns to the upload of candidate k + 1 (if it is not resident): into
+            // the buffer join k - 1 read, behind that join, while join k runs.  (An upload from pageable memory
+            // holds the host until it is through, so it must not come before the join it overlaps is queued.)
+            if (next == k + 1 && next < order.size()) {
+                upload(*spare[(next - 1) % 2], order[next]);
+                ++next;
             }
-            HIP_CHECK(hipStreamSynchronize(dev.compute));
-            unsigned long long after = 0;
-            HIP_CHECK(hipMemcpy(&after, g_ws.counters, sizeof after, hipMemcpyDeviceToHost));
-            HIP_CHECK(fasted::launch_offset_pairs(dPairs, std::min(before, devCap), std::min(after, devCap),
-                                                  (int)(i * rows), (int)(j * rows), dev.compute));
-            before = after;
         }
+        HIP_CHECK(hipEventRecord(query->released, dev.compute));
+        HIP_CHECK(hipStreamSynchronize(dev.compute));
+        unsigned long long before = 0;
+        HIP_CHECK(hipMemcpy(&before, g_ws.counters, sizeof before, hipMemcpyDeviceToHost));
         const unsigned long long kept = std::min(before, devCap);
         if (kept > 1) HIP_CHECK(fasted::sort_pairs_row_major(dPairs, kept, dev.compute, &g_sortWs, n, n));
         HIP_CHECK(hipStreamSynchronize(dev.compute));
@@ -459,6 +562,16 @@ void self_join_blocked(const uint16_t* points, long long n, int d, double epsilo
             HIP_CHECK(hipMemcpy(out + storedAll, dPairs, (size_t)take * sizeof(FastedPair), hipMemcpyDeviceToHost));
         storedAll += take;
         foundAll += before;
+        // roles for query block i + 1: its rows are in the buffer read last; the old query block stays resident
+        if (i + 1 < blocks) {
+            const size_t lastPos = order.size() - 1;
+            BlockBuffer* const last = spare[(lastPos - 1) % 2];
+            BlockBuffer* const other = spare[lastPos % 2];
+            if (last->block != i + 1) throw std::logic_error("blocked join: the next query block is not resident");
+            spare[0] = query;
+            spare[1] = other;
+            query = last;
+        }
     }
     if (found) *found = foundAll;
     if (stored) *stored = storedAll;
@@ -636,15 +749,7 @@ unsigned long long ensure_pair_buffer(int n) {
         g_pairWs.capPairs = 0;
     }
     g_sortWs.release();
-    size_t freeB = 0, totalB = 0;
-    HIP_CHECK(hipMemGetInfo(&freeB, &totalB));
-    const size_t usable = freeB - freeB / 16;  // leave some room for the runtime
-    unsigned long long maxPairs = want;
-    for (int round = 0; round < 4; ++round) {
-        const size_t need = (size_t)maxPairs * sizeof(FastedPair) + fasted::sort_scratch_bytes(maxPairs);
-        if (need <= usable) break;
-        maxPairs = (unsigned long long)((double)maxPairs * (double)usable / (double)need * 0.98);
-    }
+    const unsigned long long maxPairs = fit_pairs_with_sort(want);
     if (maxPairs < want)
         std::printf("Failed to allocate enough space for %llu pairs. Reducing max number of pairs to %llu\n", want, maxPairs);
     HIP_CHECK(hipMalloc(&g_pairWs.dPairs, (size_t)(maxPairs ? maxPairs : 1) * sizeof(FastedPair)));
@@ -1195,6 +1300,14 @@ const FastedPair* fasted_last_pairs_device(unsigned long long* stored) {
 
 const char* fasted_last_error(void) { return g_error.c_str(); }
 
-const char* fasted_version(void) { return "fasted-mi355x 0.1 (gfx950)"; }
+const char* fasted_version(void) {
+    static const std::string version = [] {
+        std::string v = "fasted-mi355x 0.1 (gfx950)";
+        const char* const tag = fasted::build_tag();
+        if (tag[0]) v += std::string(" ") + tag;
+        return v;
+    }();
+    return version.c_str();
+}
 
 }  // extern "C"

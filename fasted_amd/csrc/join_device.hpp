@@ -12,10 +12,12 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Counter block of one join: word 0 = pairs found, word 1 = non-finite flag, then the 8 queue heads, each on
-// its own 128-byte line.
+// Counter block of one join: word 0 = pairs found, word 1 = non-finite flag, words 2 and 3 = clock readings,
+// then the 8 queue heads, each on its own 128-byte line.
 constexpr int kCounterFound = 0;
-constexpr int kCounterNonFinite = 1;  // non-zero: some point of the join has a non-finite squared norm
+constexpr int kCounterNonFinite = 1;  // == the join's epoch: some point of the join has a non-finite squared norm
+constexpr int kCounterStampNorms = 2;  // the device's constant-rate clock when the join's first norm kernel started
+constexpr int kCounterStampJoin = 3;   // ... when the join kernel started
 constexpr int kQueueBase = 16, kQueueStride = 16;
 constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
 
@@ -31,6 +33,7 @@ struct JoinParams {
     const float* halfQ;  // per query point: eps^2/4 - s/2, s = squared norm
     const float* halfC;  // ... per candidate point
     unsigned long long* counters;
+    unsigned long long epoch;  // number of this join (never 0): the value of the non-finite flag that counts
     int2* pairs;
     unsigned long long cap;
     TileOrder raster;

@@ -22,7 +22,9 @@ struct JoinLaunch {
     int dPad;                    // K extent, multiple of kSlabK
     const float* halfQ;          // per query point: eps^2/4 - s/2 (s = squared norm), see launch_sum_squared
     const float* halfC;          // ... per candidate point
-    unsigned long long* counters;  // counter_words() words: [0] pairs found, then the queue heads
+    unsigned long long* counters;  // counter_words() words: [0] pairs found, [1] non-finite flag, then the queue heads
+    unsigned long long epoch = 1;  // number of the join: what the norm kernels of THIS join write into the
+                                   // non-finite flag (a flag left by an earlier join is not seen)
     void* pairs;                 // FastedPair[cap]
     unsigned long long cap;
     bool epilogue;               // false: contraction only (measurement)
@@ -40,21 +42,32 @@ int lds_chunk_slot(int row, int chunk);
 // Squared norms of n points into `sums` (may be null) and, when `halves` is given, the per-point start value of
 // the join's accumulators  h = eps2/4 - s/2  (eps2 = (float)(eps*eps), source/findPairs.cuh:678): the join kernel
 // tests  h_q + h_c + q.c >= 0.  A non-finite norm raises the flag in `counters` (the join then tests element
-// by element), so the counters must have been reset before.
+// by element): the flag word receives `epoch`.  With `reset` the kernel also clears the pair counter and the
+// queue heads for the join that follows (no launch_reset_counters needed).
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, float* halves, float eps2,
-                              unsigned long long* counters, hipStream_t stream);
+                              unsigned long long* counters, hipStream_t stream, unsigned long long epoch = 1,
+                              bool reset = false);
 // The same halves from norms that are already there.
 hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, unsigned long long* counters,
-                         hipStream_t stream);
+                         hipStream_t stream, unsigned long long epoch = 1, bool reset = false);
 // *badRows += number of rows whose columns d .. dPad-1 are not all zeros.
 hipError_t launch_padding_check(const void* points, long long ld, int n, int d, int dPad, unsigned long long* badRows,
                                 hipStream_t stream);
-// Clears the queue heads and, unless keepFound, the pair counter and the non-finite flag (words 0, 1 of `counters`).
+// Clears the queue heads and, unless keepFound, the pair counter (word 0 of `counters`).
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream);
+// hostWords (pinned host memory, device-visible address) [0] = the pair counter, [1], [2] = the constant-rate clock
+// at the start of the join's first norm kernel and of the join kernel, [3] = now; written by a one-thread kernel.
+hipError_t launch_publish_count(const unsigned long long* counters, unsigned long long* hostWords, hipStream_t stream);
 // pairs[first, last): QueryPoint += qOffset, CandidatePoint += cOffset.
 hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,
                                hipStream_t stream);
+// The same for the pairs [min(mark[0], cap), min(counter, cap)) that the join before this launch appended; leaves
+// the counter in mark[1].  No host round trip: the range is read on the device.
+hipError_t launch_offset_appended_pairs(void* pairs, unsigned long long* mark, const unsigned long long* counters,
+                                        unsigned long long cap, int qOffset, int cOffset, hipStream_t stream);
 hipError_t launch_join(const JoinLaunch& p, hipStream_t stream);
+// "" for the library proper; a measurement build of the join kernel (parts compiled out) names itself here.
+const char* build_tag();
 
 
 // Device buffers of the row-major sort (a second key buffer and the radix sort's own storage).  They only

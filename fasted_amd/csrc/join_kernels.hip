@@ -59,6 +59,8 @@ constexpr int kWaveCols = 64;                       // columns of a wave's outpu
 //                 bit 1: no global -> LDS transfers once both LDS stages hold the first two slabs of the
 //                        workgroup's first tile (the matrix cores keep seeing real operand values)
 //                 bit 2: no LDS fragment reads (the operand registers hold whatever they held)
+//                 bit 3: the hit bits of a tile are formed but no pair is extracted from them
+//                 bit 4: only the screening of a tile (is there any hit in the wave?), no hit bits, no pairs
 //   FASTED_ABLATE_PANELS k > 0: every tile reads the panels (row % k, col % k): the whole join touches
 //                        k panels of 256 points only, so they stay in the Infinity Cache (or the L2)
 #ifndef FASTED_ABLATE
@@ -68,7 +70,8 @@ constexpr int kWaveCols = 64;                       // columns of a wave's outpu
 #define FASTED_ABLATE_PANELS 0
 #endif
 constexpr bool kNoInit = (FASTED_ABLATE & 1) != 0, kNoTransfers = (FASTED_ABLATE & 2) != 0,
-               kNoFragments = (FASTED_ABLATE & 4) != 0;
+               kNoFragments = (FASTED_ABLATE & 4) != 0, kNoExtract = (FASTED_ABLATE & 24) != 0,
+               kNoHits = (FASTED_ABLATE & 16) != 0;
 __device__ __forceinline__ unsigned panel_of(unsigned tile) {
     return FASTED_ABLATE_PANELS > 0 ? tile % (unsigned)(FASTED_ABLATE_PANELS > 0 ? FASTED_ABLATE_PANELS : 1) : tile;
 }
@@ -125,11 +128,23 @@ inline void raster_decode(const Raster& r, bool tall, unsigned q, unsigned long 
 
 // ------------------------------------------------------------------------------------------
 // Optionally also writes, per point, h = quarterEps2 - s/2 (what the join kernel starts its accumulators
-// from) and raises the non-finite flag of the counter block when a squared norm is infinite or NaN.
+// from) and raises the non-finite flag of the counter block when a squared norm is infinite or NaN: the flag
+// word receives `epoch`, the number of the join this launch belongs to, so that it never has to be cleared
+// (clearing it in this kernel would race with raising it).  With `reset`, the first workgroup clears the pair
+// counter and the queue heads for the join kernel that follows in the stream: no launch of its own for that.
+__device__ __forceinline__ void reset_for_join(unsigned long long* __restrict__ counters) {
+    if (blockIdx.x != 0) return;
+    const int t = threadIdx.x;
+    if (t == 0) counters[kCounterStampNorms] = wall_clock64();  // the timed region of a small join starts here
+    if (t < kCounterWords && t != kCounterNonFinite && t != kCounterStampNorms && t != kCounterStampJoin) counters[t] = 0ull;
+}
+
 __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restrict__ pts, long long ld16, int n,
                                                           int chunksPerRow, int lanesPerRow,
                                                           float* __restrict__ sums, float* __restrict__ halves,
-                                                          float quarterEps2, unsigned long long* __restrict__ counters) {
+                                                          float quarterEps2, unsigned long long* __restrict__ counters,
+                                                          unsigned long long epoch, int reset) {
+    if (reset) reset_for_join(counters);
     const int lane = threadIdx.x & 63;
     const long long wave = ((long long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int rowsPerWave = 64 / lanesPerRow;
@@ -169,19 +184,21 @@ __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restric
         if (sums) sums[row] = acc;
         if (halves) {
             halves[row] = __builtin_fmaf(acc, -0.5f, quarterEps2);
-            if (!(__builtin_fabsf(acc) < __builtin_inff())) counters[kCounterNonFinite] = 1ull;
+            if (!(__builtin_fabsf(acc) < __builtin_inff())) counters[kCounterNonFinite] = epoch;
         }
     }
 }
 
 // The same per-point halves from squared norms that are already there.
 __global__ void __launch_bounds__(256) halves_kernel(const float* __restrict__ sums, int n, float quarterEps2,
-                                                     float* __restrict__ halves, unsigned long long* __restrict__ counters) {
+                                                     float* __restrict__ halves, unsigned long long* __restrict__ counters,
+                                                     unsigned long long epoch, int reset) {
+    if (reset) reset_for_join(counters);
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float s = sums[i];
     halves[i] = __builtin_fmaf(s, -0.5f, quarterEps2);
-    if (!(__builtin_fabsf(s) < __builtin_inff())) counters[kCounterNonFinite] = 1ull;
+    if (!(__builtin_fabsf(s) < __builtin_inff())) counters[kCounterNonFinite] = epoch;
 }
 
 // Rows whose padding columns d .. dPad-1 hold anything but zeros (the kernels read them unmasked, so they must
@@ -196,17 +213,50 @@ __global__ void __launch_bounds__(256) padding_check_kernel(const unsigned short
     if (bad) atomicAdd(badRows, 1ull);
 }
 
-// Clears the queue heads and, unless `keepFound`, the pair counter (word 0) and the non-finite flag (word 1):
-// a launch that keeps them appends its pairs behind those of the launch before.
+// Clears the queue heads and, unless `keepFound`, the pair counter (word 0): a launch that keeps it appends its
+// pairs behind those of the launch before.  The non-finite flag (word 1) is never cleared: it holds the number
+// of the join that raised it.  (A join that computes its norms first needs no launch of this: the norm kernel's
+// first workgroup does the clearing.)
 __global__ void reset_counters_kernel(unsigned long long* c, int keepFound) {
-    if (threadIdx.x < kCounterWords && !(keepFound && (threadIdx.x == kCounterFound || threadIdx.x == kCounterNonFinite)))
+    if (threadIdx.x < kCounterWords && threadIdx.x != kCounterNonFinite && !(keepFound && threadIdx.x == kCounterFound))
         c[threadIdx.x] = 0ull;
+}
+
+// Copies the pair counter and the clock readings of the norm and join kernels into pinned host memory that the
+// device can write, and adds its own reading: it starts when the join kernel is over.  (A one-thread kernel behind
+// the join is no slower than a copy command of a few bytes, and its clock reading replaces an event.)
+__global__ void publish_count_kernel(const unsigned long long* __restrict__ counters, unsigned long long* hostWords) {
+    const unsigned long long now = wall_clock64();
+    hostWords[0] = counters[kCounterFound];
+    hostWords[1] = counters[kCounterStampNorms];
+    hostWords[2] = counters[kCounterStampJoin];
+    hostWords[3] = now;
+    __threadfence_system();
 }
 
 // Adds the first row of the query block and of the candidate block to the pairs [first, last) that a
 // join of two row blocks of a larger dataset has appended with block-local indices.
 __global__ void __launch_bounds__(256) offset_pairs_kernel(int2* pairs, unsigned long long first,
                                                            unsigned long long last, int qOffset, int cOffset) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = first + (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < last; i += stride) {
+        int2 v = pairs[i];
+        v.x += qOffset;
+        v.y += cOffset;
+        pairs[i] = v;
+    }
+}
+
+// The same for the pairs a join has just appended, with the range taken from device memory, so that a series of
+// block joins needs no host round trip in between: the range starts at *mark (where the join before this one
+// ended; the caller zeroes the first mark) and ends at the pair counter, both clipped to the capacity; the
+// counter is then left in mark[1] for the launch after the next join.
+__global__ void __launch_bounds__(256) offset_appended_pairs_kernel(int2* pairs, unsigned long long* mark,
+                                                                    const unsigned long long* __restrict__ counters,
+                                                                    unsigned long long cap, int qOffset, int cOffset) {
+    const unsigned long long found = counters[kCounterFound];
+    const unsigned long long first = mark[0] < cap ? mark[0] : cap, last = found < cap ? found : cap;
+    if (blockIdx.x == 0 && threadIdx.x == 0) mark[1] = found;
     const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
     for (unsigned long long i = first + (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < last; i += stride) {
         int2 v = pairs[i];
@@ -274,8 +324,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // two slots of [0] row, [1] col
     const int2* const sStage = reinterpret_cast<const int2*>(lds + kLdsStage) + wave * kWaveStagePairs;  // this wave's region
 
-    // set by the kernel that formed the per-point halves: some point has a non-finite squared norm
-    const bool nonFinite = p.counters[kCounterNonFinite] != 0ull;
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.counters[kCounterStampJoin] = wall_clock64();  // (timing of small joins)
+
+    // set by the kernel that formed this join's per-point halves: some point has a non-finite squared norm
+    const bool nonFinite = p.counters[kCounterNonFinite] == p.epoch;
 
     // Which XCD this workgroup runs on (hardware register XCC_ID, low 3 bits).
     // (thread 0 moves on to the queue it last found work in once its own is exhausted)
@@ -677,7 +729,8 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
                 for (int fi = 1; fi < kFragRows; ++fi) best = __builtin_fmaxf(best, rowBest[fi]);
                 any = __builtin_amdgcn_ballot_w64(best >= 0.0f) != 0ull;
-                if (any) {
+                if (kNoHits) asm volatile("" ::"v"(best));
+                if (any && !kNoHits) {
                     // the rows of blocks with a hit somewhere in the wave yield their bits, one instruction per
                     // element: the sign of the accumulator (set = no hit) is shifted in.  (The eight compares are
                     // issued together: one at a time, each branch waits for its compare.)
@@ -729,7 +782,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                     hits[fp] = m;
                 }
             }
-            if (any) {
+            if (kNoExtract) {
+                if (any && !kNoHits) {
+#pragma unroll
+                    for (int fp = 0; fp < kFragRows / 2; ++fp) asm volatile("" ::"v"(hits[fp]));
+                }
+            } else if (any) {
                 // Extraction.  A round takes the first remaining hit of every lane that has one in a word of hit
                 // bits: the lanes form a mask in scalar registers, a lane's record goes behind those of the lanes
                 // before it, the wave's fill count moves on by the number of lanes.
@@ -843,6 +901,15 @@ int raster_coord(unsigned long long idx, long long nQ, long long nC, bool upperO
 
 int counter_words() { return kCounterWords; }
 
+// "" for the library proper; a measurement build names what it leaves out (its results are wrong by construction)
+#define FASTED_STR2(x) #x
+#define FASTED_STR(x) FASTED_STR2(x)
+const char* build_tag() {
+    return (FASTED_ABLATE != 0 || FASTED_ABLATE_PANELS != 0)
+               ? "ABLATION BUILD (ablate=" FASTED_STR(FASTED_ABLATE) ", panels=" FASTED_STR(FASTED_ABLATE_PANELS) "): results are wrong by construction"
+               : "";
+}
+
 unsigned long long tile_count(long long nQ, long long nC) {
     const Raster r = make_raster(nQ, nC);
     return (unsigned long long)r.tileRows * r.tileCols;
@@ -850,11 +917,14 @@ unsigned long long tile_count(long long nQ, long long nC) {
 
 int lds_chunk_slot(int row, int chunk) { return (chunk ^ swz(row)) & 7; }
 
-// (float)(eps*eps) / 4, kept finite: the kernels rely on finite accumulator start values
-float quarter_eps2(float eps2) { return (eps2 < 3.0e38f ? eps2 : 3.0e38f) * 0.25f; }
+// (float)(eps*eps) / 4, kept finite: the kernels rely on finite accumulator start values, so an infinite
+// epsilon (every pair of finite points is a hit) is clamped.  The host entries refuse a NaN epsilon; should one
+// arrive here all the same, the start values become hugely negative: no distance passes the test, as no
+// distance compares <= NaN in the reference (source/warpMma.cuh:257), and only the forced self pairs remain.
+float quarter_eps2(float eps2) { return (eps2 != eps2 ? -3.0e38f : (eps2 > 3.0e38f ? 3.0e38f : eps2)) * 0.25f; }
 
 hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad, float* sums, float* halves, float eps2,
-                              unsigned long long* counters, hipStream_t stream) {
+                              unsigned long long* counters, hipStream_t stream, unsigned long long epoch, bool reset) {
     const int chunksPerRow = dPad / 8;
     int lanesPerRow = 64;
     while (lanesPerRow > chunksPerRow) lanesPerRow >>= 1;
@@ -863,13 +933,14 @@ hipError_t launch_sum_squared(const void* points, long long ld, int n, int dPad,
     const long long blocks = (waves + 3) / 4;
     sum_squared_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(static_cast<const u32x4*>(points), ld / 8, n,
                                                                         chunksPerRow, lanesPerRow, sums, halves,
-                                                                        quarter_eps2(eps2), counters);
+                                                                        quarter_eps2(eps2), counters, epoch, reset ? 1 : 0);
     return hipGetLastError();
 }
 
 hipError_t launch_halves(const float* sums, int n, float eps2, float* halves, unsigned long long* counters,
-                         hipStream_t stream) {
-    halves_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(sums, n, quarter_eps2(eps2), halves, counters);
+                         hipStream_t stream, unsigned long long epoch, bool reset) {
+    halves_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(sums, n, quarter_eps2(eps2), halves, counters,
+                                                                               epoch, reset ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -886,6 +957,11 @@ hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, h
     return hipGetLastError();
 }
 
+hipError_t launch_publish_count(const unsigned long long* counters, unsigned long long* hostWords, hipStream_t stream) {
+    publish_count_kernel<<<1, 1, 0, stream>>>(counters, hostWords);
+    return hipGetLastError();
+}
+
 hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,
                                hipStream_t stream) {
     if (last <= first || (qOffset == 0 && cOffset == 0)) return hipSuccess;
@@ -895,59 +971,27 @@ hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned l
     return hipGetLastError();
 }
 
-hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
-    static int numCUs = 0;
-    static bool configured = false;
-    if (!configured) {
-        int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
-        if (e != hipSuccess) return e;
-        hipDeviceProp_t prop;
-        e = hipGetDeviceProperties(&prop, dev);
-        if (e != hipSuccess) return e;
-        numCUs = prop.multiProcessorCount;
-        configured = true;
-    }
-    const JoinLaunch& l = launch;
-    JoinParams p;
-    p.ptsQ = static_cast<const u32x4*>(l.queries);
-    p.ptsC = static_cast<const u32x4*>(l.candidates);
-    p.ldQ16 = l.ldQ / 8;
-    p.ldC16 = l.ldC / 8;
-    p.nQ = l.nQ;
-    p.nC = l.nC;
-    p.selfStride = l.forcedStride > 0 ? l.forcedStride : (l.selfJoin ? 1 : 0);
-    p.symmetric = (l.selfJoin && l.symmetric) ? 1 : 0;
-    p.nSlabs = l.dPad / kSlabK;
-    p.halfQ = l.halfQ;
-    p.halfC = l.halfC;
-    p.counters = l.counters;
-    p.pairs = static_cast<int2*>(l.pairs);
-    p.cap = l.cap;
-    // Tiles of 128 query rows when the matrix then still has no more tiles than the chip has workgroups (never
-    // in symmetric mode, whose diagonal logic assumes square tiles): twice as many workgroups work, each on half a
-    // tile.  A 128-row tile costs about 0.7 of a 256-row one (64 x 64 wave sub-tiles need a third more LDS fragment
-    // reads per MFMA), so the finer grid only pays while it fits one round: measured on Exp(40) data, 1000 and 2154
-    // points 1.1x - 1.4x faster, 3000 points (288 tiles of 128 rows: two rounds) 1.4x slower.
-    // FASTED_TILE_ROWS=256 or 128 in the environment overrides the choice (tests run both).
-    const unsigned long long tiles128 = (unsigned long long)((l.nQ + 127) / 128) * ((l.nC + kTile - 1) / kTile);
-    bool rows128 = p.symmetric == 0 && tiles128 <= (unsigned long long)numCUs;
-    const char* const forced = getenv("FASTED_TILE_ROWS");  // read at every launch: a test sets it per case
-    const int forcedRows = forced ? atoi(forced) : 0;
-    if (forcedRows == 256) rows128 = false;
-    if (forcedRows == 128 && p.symmetric == 0) rows128 = true;
-    const int tileRows = rows128 ? 128 : kTile;
-    p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0, tileRows);
-    unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
+hipError_t launch_offset_appended_pairs(void* pairs, unsigned long long* mark, const unsigned long long* counters,
+                                        unsigned long long cap, int qOffset, int cOffset, hipStream_t stream) {
+    offset_appended_pairs_kernel<<<dim3(512), dim3(256), 0, stream>>>(static_cast<int2*>(pairs), mark, counters, cap, qOffset,
+                                                                     cOffset);
+    return hipGetLastError();
+}
+
+namespace {
+
+// One launch of the join kernel over the tile grid described by p.raster, in the queue or the direct mode, with
+// tiles of 256 or 128 query rows.
+hipError_t launch_join_grid(JoinParams p, bool rows128, bool tall, bool epilogue, int numCUs, hipStream_t stream) {
+    const unsigned long long realTiles = (unsigned long long)p.raster.tileRows * p.raster.tileCols;
     // Up to two tiles per CU, workgroup b computes tile b and ends, one workgroup per tile (the hardware places
     // the second round as CUs fall free); from there on, one persistent workgroup per CU draws from the queues.
     p.direct = realTiles <= 2ull * (unsigned long long)numCUs ? 1 : 0;
     unsigned grid = (unsigned)(p.direct ? realTiles : (unsigned long long)numCUs);
     if (grid == 0) grid = 1;
-    const bool tall = tall_order(l.nQ, tileRows);
     const dim3 g(grid), b(kThreads);
     const bool oneSlab = p.nSlabs == 1;
-    const int variant = (oneSlab ? 8 : 0) | (l.epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
+    const int variant = (oneSlab ? 8 : 0) | (epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
     switch (variant) {
         case 15: join_kernel<true, true, 128, true><<<g, b, 0, stream>>>(p); break;
         case 14: join_kernel<true, true, 256, true><<<g, b, 0, stream>>>(p); break;
@@ -967,6 +1011,49 @@ hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
         default: join_kernel<false, false, 256, false><<<g, b, 0, stream>>>(p); break;
     }
     return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_join(const JoinLaunch& launch, hipStream_t stream) {
+    // (the compute units of the current device, looked up at every launch: the device may change between calls)
+    int dev = 0, numCUs = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&numCUs, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    const JoinLaunch& l = launch;
+    JoinParams p;
+    p.ptsQ = static_cast<const u32x4*>(l.queries);
+    p.ptsC = static_cast<const u32x4*>(l.candidates);
+    p.ldQ16 = l.ldQ / 8;
+    p.ldC16 = l.ldC / 8;
+    p.nQ = l.nQ;
+    p.nC = l.nC;
+    p.selfStride = l.forcedStride > 0 ? l.forcedStride : (l.selfJoin ? 1 : 0);
+    p.symmetric = (l.selfJoin && l.symmetric) ? 1 : 0;
+    p.nSlabs = l.dPad / kSlabK;
+    p.halfQ = l.halfQ;
+    p.halfC = l.halfC;
+    p.counters = l.counters;
+    p.epoch = l.epoch;
+    p.pairs = static_cast<int2*>(l.pairs);
+    p.cap = l.cap;
+    // Tiles of 128 query rows when the matrix then still has no more tiles than the chip has workgroups (never
+    // in symmetric mode, whose diagonal logic assumes square tiles): twice as many workgroups work, each on half a
+    // tile.  A 128-row tile costs about 0.7 of a 256-row one (64 x 64 wave sub-tiles need a third more LDS fragment
+    // reads per MFMA), so the finer grid only pays while it fits one round: measured on Exp(40) data, 1000 and 2154
+    // points 1.1x - 1.4x faster, 3000 points (288 tiles of 128 rows: two rounds) 1.4x slower.
+    // FASTED_TILE_ROWS=256 or 128 in the environment overrides the choice (tests run both).
+    const unsigned long long tiles128 = (unsigned long long)((l.nQ + 127) / 128) * ((l.nC + kTile - 1) / kTile);
+    bool rows128 = p.symmetric == 0 && tiles128 <= (unsigned long long)numCUs;
+    const char* const forced = getenv("FASTED_TILE_ROWS");  // read at every launch: a test sets it per case
+    const int forcedRows = forced ? atoi(forced) : 0;
+    if (forcedRows == 256) rows128 = false;
+    if (forcedRows == 128 && p.symmetric == 0) rows128 = true;
+    const int tileRows = rows128 ? 128 : kTile;
+    p.raster = make_raster(l.nQ, l.nC, p.symmetric != 0, tileRows);
+    return launch_join_grid(p, rows128, tall_order(l.nQ, tileRows), l.epilogue, numCUs, stream);
 }
 
 }  // namespace fasted

@@ -124,3 +124,145 @@ class SweepDriver:
                 records += self.timed_runs(target, epsilon, 1)
             by_dataset[Path(path).name] = records
         return self.write(prefix, by_dataset)
+
+
+# ---- the reference runner's names ------------------------------------------------------------------------
+# Scripts written against results/scripts/experiment/experiments.py (run_experiments.py of the reference builds
+# an ``ExperimentRunner(load_findpairs())`` and calls the methods below) keep working on this package: same
+# class, method and argument names, same result files.  Everything is carried out by a ``SweepDriver`` over a
+# backend that wraps the object handed in -- the loaded library or a mock with the same three methods
+# (``runFromExponentialDataset``, ``runFromFile``, ``reRun``; results/scripts/tests/test_experiments.py:14-71).
+from dataclasses import dataclass  # noqa: E402
+
+
+@dataclass
+class SearchParameters:
+    """One timed configuration (experiments.py:58-64)."""
+    target_selectivity: float
+    epsilon: float
+    save_pairs: bool
+
+
+@dataclass
+class Experiment:
+    """One result record (experiments.py:67-73)."""
+    selectivity: float
+    epsilon: float
+    iteration: int
+    results: object
+
+
+class ResultsEncoder(json.JSONEncoder):
+    """Writes ``Experiment`` records and ``Results`` structures as the reference's files hold them."""
+
+    def default(self, obj):
+        if isinstance(obj, Experiment):
+            return {"selectivity": obj.selectivity, "epsilon": obj.epsilon, "iteration": obj.iteration,
+                    "results": results_record(obj.results)}
+        if hasattr(obj, "pairsFound") and hasattr(obj, "inputProblemShape"):
+            return results_record(obj)
+        return super().default(obj)
+
+
+def find_epsilon_binary(target_selectivity, get_selectivity, initial_epsilon=0.0):
+    """Epsilon whose selectivity lies within 1 % of the target, for any ``get_selectivity(epsilon)`` callable:
+    the procedure of the library's native search (``fasted_find_epsilon``), which is the reference's
+    (experiments.py:228-281) -- double from the initial epsilon (0 -> 2) until the target is passed, then half
+    steps -- with its guard against a plateau."""
+    low = high = float(initial_epsilon)
+    seen = 0.0
+    while seen < target_selectivity:
+        low, high = high, (2.0 if high == 0.0 else 2.0 * high)
+        if high > 100000.0:
+            raise ValueError(f"no epsilon up to 100000 reaches a selectivity of {target_selectivity}")
+        seen = get_selectivity(high)
+    previous, epsilon = high, 0.5 * (low + high)
+    seen = get_selectivity(epsilon)
+    for _ in range(200):
+        if abs(seen - target_selectivity) / target_selectivity < 0.01:
+            return epsilon
+        half_step = 0.5 * abs(epsilon - previous)
+        previous, epsilon = epsilon, (epsilon - half_step if seen > target_selectivity else epsilon + half_step)
+        if epsilon == previous:
+            break
+        seen = get_selectivity(epsilon)
+    raise ValueError("epsilon search did not converge to within 1% of the target selectivity")
+
+
+class _CallableBackend:
+    """Backend over the three entry points of a pair-finding object (the loaded library or a mock)."""
+
+    def __init__(self, find_pairs):
+        self._fp = find_pairs
+        self._first = None  # the loading call that a run on fresh data makes
+
+    def load_exponential(self, size, dim, lam=40.0, value_range=10.0):
+        self._first = lambda eps, save: self._fp.runFromExponentialDataset(int(size), int(dim), lam, value_range, eps, save)
+
+    def load_file(self, path):
+        self._first = lambda eps, save: self._fp.runFromFile(str(path).encode("utf-8"), eps, save)
+
+    def run(self, epsilon, save_pairs=False):
+        first, self._first = self._first, None
+        return first(epsilon, save_pairs) if first else self._fp.reRun(epsilon, save_pairs)
+
+    def epsilon_for(self, target, sample_rows=None):
+        probes = []
+
+        def selectivity(eps):
+            probes.append(eps)
+            return self.run(eps, False).get_selectivity()
+
+        eps = find_epsilon_binary(target, selectivity)
+        return eps, selectivity(eps), len(probes)
+
+
+class ExperimentRunner:
+    """The reference's runner (experiments.py:341-591) by name; the work is a ``SweepDriver``'s."""
+
+    def __init__(self, find_pairs, output_dir="."):
+        self._find_pairs = find_pairs
+        self._driver = SweepDriver(_CallableBackend(find_pairs), output_dir)
+
+    def get_selectivity_rerun(self, epsilon):
+        return self._find_pairs.reRun(epsilon, False).get_selectivity()
+
+    def run_time_trials(self, find_pairs, search_params, iterations):
+        out = []
+        for p in search_params:
+            for i in range(iterations):
+                try:
+                    out.append(Experiment(p.target_selectivity, p.epsilon, i, find_pairs(p.epsilon, p.save_pairs and i == 0)))
+                except Exception as e:  # noqa: BLE001
+                    print(f"Failed to run iteration {i}. {e}")
+        return out
+
+    def run_selectivity_experiment(self, selectivities, find_pairs, iterations=3, save_pairs=False):
+        out = []
+        for target in selectivities:
+            eps = find_epsilon_binary(target, lambda e: find_pairs(e, False).get_selectivity())
+            out += self.run_time_trials(find_pairs, [SearchParameters(target, eps, save_pairs)], iterations)
+        return out
+
+    def build_file_pairs_finder(self, base_path, dataset):
+        path = str(Path(base_path) / dataset).encode("utf-8")
+        return lambda epsilon, save_pairs: self._find_pairs.runFromFile(path, epsilon, save_pairs)
+
+    def build_rerunnable_file_pairs_finder(self, base_path, dataset):
+        return fp.RerunnablePairsFinder(self.build_file_pairs_finder(base_path, dataset), self._find_pairs.reRun)
+
+    def run_real_dataset_known_epsilons_experiments(self, dataset_path, dataset, search_params, num_repetitions=3):
+        runs = [(p.target_selectivity, p.epsilon) for p in search_params]
+        save = any(p.save_pairs for p in search_params)
+        return self._driver.file_runs(Path(dataset_path) / dataset, runs, num_repetitions, save, prefix=f"{dataset}_results")
+
+    def run_real_datasets_epsilon_finder_experiments(self, target_selectivities, base_path=".", datasets=()):
+        """The reference lists its datasets and their directory in the method body (experiments.py:497-508);
+        here they are arguments."""
+        return self._driver.file_epsilon_search([Path(base_path) / d for d in datasets], target_selectivities)
+
+    def run_selectivity_vs_speed_experiment(self, target_selectivities):
+        return self._driver.selectivity_sweep(target_selectivities)
+
+    def run_speed_sweeps_exponential_data_experiment(self):
+        return self._driver.exponential_sweep()

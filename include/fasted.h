@@ -70,9 +70,13 @@ void releaseResources(void);
 /* ---- group 2: raw buffers ----------------------------------------------------------
  * Return 0 on success, non-zero on failure; fasted_last_error() then describes it.     */
 
+/* The two kernel times are HIP-event times on the stream, as the reference measures them
+ * (source/findPairs.cuh:625-639,695-697); for joins of at most 512 tiles of 256 x 256, where three event records
+ * would cost a third of the call, they are differences of the device's constant-rate clock, read by the kernels
+ * themselves as they start (hipDeviceAttributeWallClockRate ticks). */
 typedef struct FastedJoinStats {
-    float sumSquaredMs; /* HIP-event time of counter reset + squared-norm pre-pass */
-    float joinMs;       /* HIP-event time of the join kernel */
+    float sumSquaredMs; /* squared-norm pre-pass (which also clears the counters): its start to the join kernel's start */
+    float joinMs;       /* the join kernel: its start to the start of what follows it on the stream */
     float sortMs;       /* host wall time of the row-major sort, stream synchronisation included (0 when not sorted) */
     int paddedN;        /* rows covered by the tile grid */
     int paddedD;        /* K extent the kernel looped over */
@@ -104,8 +108,10 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
 
 /* The same join for a dataset that does not fit the device (or should not occupy it): the host-resident
  * points are streamed through the device in blocks of `block_rows` points (rounded up to a multiple of
- * 256).  Device memory used: three blocks, their norms, and a pair buffer of min(cap, block_rows*256)
- * records (twice that while sorting).  Output as fasted_self_join: row-major, *found counts every pair,
+ * 256).  Device memory used: three blocks, 4 bytes per point of the whole dataset (each point's squared norm
+ * enters the join through one float, formed when its block is first uploaded), and a pair buffer of
+ * min(cap, block_rows*256) records (about three times that while sorting).  Blocks that a later join still
+ * needs stay on the device: with B blocks about B*(B-2)+2 block uploads instead of B*B.  Output as fasted_self_join: row-major, *found counts every pair,
  * at most `cap` are written; in addition the pairs of one block of query points beyond block_rows*256 are
  * counted but not written.  The reference has no such path: its dataset, twice, and N*256 pair records
  * must fit the device (source/findPairs.cuh:568-600,644-647); "batching" is named as future work in its
@@ -122,15 +128,21 @@ int fasted_self_join_blocked(const uint16_t* points, long long n, int d, double 
  *              workspace is used)
  *   d_pairs    room for `cap` pairs
  *   stream     hipStream_t (NULL = default stream)
- * The call synchronises the stream before returning and fills *stats.  Replaces the
+ * The call synchronises the stream before returning and fills *stats.  With FASTED_SORT_PAIRS the sort's
+ * device buffers (a second key buffer and the radix sort's storage, about twice the bytes of the stored
+ * pairs) are allocated by the library and kept for the next sort; so are the counters and, without d_sums,
+ * the squared norms.  releaseResources() frees all of it.  Replaces the
  * kernel launches of source/findPairs.cuh:632-687 (ComputeSquaredSums x2,
  * initOnDemandRasterizer, FindPairsKernel) and the sort of :703-704. */
 int fasted_self_join_device(const void* d_points, long long n, int d, long long ld, double epsilon, float* d_sums,
                             FastedPair* d_pairs, unsigned long long cap, unsigned flags, void* stream,
                             FastedJoinStats* stats);
 
-/* fasted_self_join_device for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The queue
+/* fasted_self_join_device for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc, programs that must not disturb a memory pool or a graph they captured elsewhere).  No
+ * counterpart in the reference.  Like fasted_self_join_device it synchronises the stream before it returns
+ * (it times itself with events and reads the pair count back), so the call itself cannot be recorded into a
+ * HIP graph capture.  The queue
  * heads, the pair counter, the squared norms and the per-point accumulator start values live in a device
  * array that is part of the library image (4 KiB + 32 MiB per GPU, held until the process ends) instead of
  * allocated workspace; the call makes no
@@ -261,6 +273,8 @@ void fasted_set_download_pairs(int enabled);
 const FastedPair* fasted_last_pairs_device(unsigned long long* stored);
 
 const char* fasted_last_error(void);
+/* Name and version of the library.  A measurement build of the join kernel (parts of it compiled out, results
+ * wrong by construction) carries the words "ABLATION BUILD" and what it leaves out in this string. */
 const char* fasted_version(void);
 
 #ifdef __cplusplus

@@ -58,6 +58,12 @@ def _load():
     lib.oracle_pair_stats.argtypes = [_i32p, _i32p, C.c_size_t, _i32p, _i32p, C.c_size_t,
                                       C.POINTER(C.c_ulonglong * 5), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.oracle_num_threads.restype = C.c_int
+    lib.oracle_blocked_join.restype = C.c_ulonglong
+    lib.oracle_blocked_join.argtypes = [_u16p, C.c_size_t, C.c_size_t, _u16p, C.c_size_t, C.c_size_t, C.c_size_t,
+                                        C.c_double, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_ulonglong,
+                                        C.POINTER(C.c_double)]
+    lib.oracle_blocked_join_vector_bits.restype = C.c_int
+    lib.oracle_blocked_join_vector_bits.argtypes = [C.c_int]
     return lib
 
 
@@ -148,6 +154,35 @@ def self_join_f32(bits, eps, n=None, sums=None):
     sums = np.ascontiguousarray(sums, dtype=np.float32)
     flat = b.reshape(-1)
     return _grow_join(lambda q, c, cap: lib().oracle_self_join_f32(flat, n, d, eps, sums, q, c, cap), 64 * n)
+
+
+def blocked_join(queries, candidates, eps, precision=64, q_offset=0, c_offset=0, want_pairs=True):
+    """The CPU baseline (oracle/blocked_join.c): cache-blocked GEMM-form join of query rows with candidate rows,
+    in FP64 or FP32.  Returns (pairs sorted row-major or None, found, seconds inside the routine)."""
+    q = np.ascontiguousarray(queries, dtype=np.uint16)
+    c = np.ascontiguousarray(candidates, dtype=np.uint16)
+    assert q.ndim == 2 and c.ndim == 2 and q.shape[1] == c.shape[1]
+    d = q.shape[1]
+    secs = C.c_double()
+    call = lambda oq, oc, cap: lib().oracle_blocked_join(  # noqa: E731
+        q.reshape(-1), q.shape[0], d, c.reshape(-1), c.shape[0], d, d, float(eps), int(precision), int(q_offset),
+        int(c_offset), oq, oc, cap, C.byref(secs))
+    if not want_pairs:
+        found = call(None, None, 0)
+        return None, int(found), secs.value
+    cap = max(1024, 64 * q.shape[0])
+    while True:
+        oq = np.empty(cap, dtype=np.int32)
+        oc = np.empty(cap, dtype=np.int32)
+        found = int(call(oq.ctypes.data, oc.ctypes.data, cap))
+        if found <= cap:
+            return sort_pairs(np.stack([oq[:found], oc[:found]], axis=1)), found, secs.value
+        cap = found
+
+
+def blocked_join_vector_bits(force=0):
+    """Vector width (256 or 512 bits) the CPU baseline runs with on this host; `force` selects one."""
+    return lib().oracle_blocked_join_vector_bits(int(force))
 
 
 def pair_distances_f64(bits, pairs):

@@ -486,3 +486,68 @@ def test_timed_runs_skip_failed_runs():
     out = ex.SweepDriver(backend).timed_runs(1, 0.5, 3, save_pairs=True)
     assert [r["iteration"] for r in out] == [0, 2]
     assert [e[1:] for e in backend.log] == [(0.5, True), (0.5, False), (0.5, False)]
+
+
+class MockLibrary:
+    """The three entry points a reference script drives (results/scripts/tests/test_experiments.py:14-71)."""
+
+    def __init__(self):
+        self.n, self.calls = 1000, []
+
+    def _results(self, eps):
+        r = fp.Results()
+        r.pairsFound = r.pairsStored = int(self.n + 50.0 * eps * self.n)
+        r.inputProblemShape.m = r.inputProblemShape.n = self.n
+        r.inputProblemShape.k = 64
+        r.TFLOPS, r.totalTime = 1.0, 0.1
+        return r
+
+    def runFromExponentialDataset(self, size, dim, lam, rng, eps, save):
+        self.calls.append(("exp", size, dim, eps, save))
+        self.n = size
+        return self._results(eps)
+
+    def runFromFile(self, path, eps, save):
+        self.calls.append(("file", path, eps, save))
+        return self._results(eps)
+
+    def reRun(self, eps, save):
+        self.calls.append(("rerun", eps, save))
+        return self._results(eps)
+
+
+def test_reference_named_runner_drives_a_mock_and_writes_the_reference_files(tmp_path):
+    """ExperimentRunner / SearchParameters / find_epsilon_binary under the reference's names
+    (results/scripts/experiment/experiments.py:58-73,228-281,341-591): a script written against them runs on
+    this package, here over a mock library; the Python search makes the probes of the restated procedure."""
+    import json
+
+    from fasted_amd import experiments as ex
+    from oracle import epsilon_search as restated
+
+    calls, calls_restated = [], []
+    sel = lambda log: (lambda e: log.append(e) or 700.0 * e ** 3)  # noqa: E731
+    assert ex.find_epsilon_binary(64, sel(calls)) == restated.find_epsilon_binary(64, sel(calls_restated))
+    assert calls == calls_restated and len(calls) > 3
+    with pytest.raises(ValueError):
+        ex.find_epsilon_binary(1e12, lambda e: 0.0)
+    with pytest.raises(ValueError):
+        ex.find_epsilon_binary(10.0, lambda e: 0.0 if e < 1.5 else 20.0)  # a step: never within 1 %
+
+    mock = MockLibrary()
+    runner = ex.ExperimentRunner(mock, output_dir=str(tmp_path))
+    path = runner.run_real_dataset_known_epsilons_experiments(str(tmp_path), "x.txt",
+                                                              [ex.SearchParameters(64, 0.5, True)], 2)
+    records = json.load(open(path))
+    assert [r["iteration"] for r in records] == [0, 1] and records[0]["epsilon"] == 0.5
+    assert set(records[0]["results"]) == {"totalTime", "TFLOPS", "pairsFound", "pairsStored", "inputProblemShape",
+                                          "paddedProblemShape"}
+    assert mock.calls[0][0] == "file" and mock.calls[0][3] is True and mock.calls[1] == ("rerun", 0.5, False)
+    path = runner.run_selectivity_vs_speed_experiment([10, 100])
+    records = json.load(open(path))
+    assert len(records) == 6 and abs(50.0 * records[0]["epsilon"] - 10) < 0.1
+    finder = runner.build_rerunnable_file_pairs_finder(str(tmp_path), "q.txt")
+    out = runner.run_selectivity_experiment([20], finder, iterations=2)
+    assert len(out) == 2 and isinstance(out[0], ex.Experiment)
+    assert json.loads(json.dumps(out, cls=ex.ResultsEncoder))[1]["iteration"] == 1
+    assert runner.get_selectivity_rerun(0.2) == pytest.approx(10.0)

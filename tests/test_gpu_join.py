@@ -471,3 +471,37 @@ def test_both_tile_heights_give_the_exact_pair_set(fasted, n, d, monkeypatch):
         monkeypatch.setenv("FASTED_TILE_ROWS", rows)
         got, st, _ = device_join(fasted, bad, eps)
         assert np.array_equal(got, want), rows
+
+
+def test_small_joins_time_themselves_with_the_device_clock(fasted):
+    """Joins of at most 512 tiles are timed by clock readings of the kernels themselves instead of events: the two
+    times must be positive, add up to less than the wall time of the call, and agree with the event-timed figure
+    of the same kernel on a matrix just large enough to be timed with events (same D, per-tile time within 2x)."""
+    import time
+
+    import torch
+
+    n, d = 4096, 128
+    bits = datasets.exponential(n, d, seed=2024)
+    eps = datasets.epsilon_for_neighbours(bits, 32)
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    cap = 300 * n
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    best = None
+    for _ in range(20):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, flags=0)
+        wall_ms = (time.perf_counter() - t0) * 1000.0
+        assert st.sumSquaredMs > 0.0 and st.joinMs > 0.0
+        assert st.sumSquaredMs + st.joinMs < wall_ms
+        best = st.joinMs if best is None else min(best, st.joinMs)
+    assert 0.003 < best < 0.2, best  # 256 tiles of two slabs: some tens of microseconds
+    # event-timed neighbour: 6000 points = 576 tiles
+    big = datasets.exponential(6000, d, seed=3)
+    ptsb = torch.from_numpy(big.view(np.int16).copy()).cuda()
+    pb = torch.empty((300 * 6000, 2), dtype=torch.int32, device="cuda")
+    tb = min(fasted.self_join_device(ptsb.data_ptr(), 6000, d, d, eps, pb.data_ptr(), pb.shape[0], flags=0).joinMs
+             for _ in range(10))
+    per_tile_small, per_tile_big = best / 1.0, tb / 3.0  # one round of the 256 workgroups against three
+    assert 0.5 < per_tile_small / per_tile_big < 2.0, (best, tb)

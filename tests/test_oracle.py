@@ -286,3 +286,55 @@ def test_pair_stats_reports_the_one_sided_pairs():
     s, diff, side = oracle.pair_stats(left, right, want_diff=True)
     assert (s["both"], s["left_only"], s["right_only"]) == (3, 1, 2)
     assert diff.tolist() == [[0, 3], [1, 2], [9, 9]] and side.tolist() == [0, 1, 1]
+
+
+# ---- the CPU baseline (oracle/blocked_join.c): a blocked GEMM-form join, pinned against the checker
+def _vector_widths():
+    native = oracle.blocked_join_vector_bits()
+    return [256, 512] if native == 512 else [256]
+
+
+@pytest.mark.parametrize("nq,nc,d", [(1, 1, 1), (7, 129, 3), (200, 333, 64), (1537, 257, 300), (50, 1000, 520)])
+def test_blocked_join_equals_the_checker(nq, nc, d):
+    """Ragged in every blocking direction (6-row panels, 128-candidate blocks, 256-wide K slices, 1536-row query
+    blocks).  Integer coordinates make both forms exact, so FP64 and FP32, 256- and 512-bit, must give exactly the
+    checker's list; indices carry the offsets handed in."""
+    from tests import datasets
+
+    bits = datasets.small_integers(nq + nc, d, high=3, seed=nq + nc + d)
+    x = bits.view(np.float16).astype(np.float64)
+    d2 = ((x[: min(nq + nc, 48), None, :] - x[None, : min(nq + nc, 48), :]) ** 2).sum(-1)
+    eps = float(np.sqrt(np.median(d2) + 0.5))
+    truth = oracle.self_join_f64(bits, eps)
+    want = truth[(truth[:, 0] < nq) & (truth[:, 1] >= nq)]
+    native = oracle.blocked_join_vector_bits()
+    try:
+        for width in _vector_widths():
+            oracle.blocked_join_vector_bits(width)
+            for precision in (64, 32):
+                got, found, secs = oracle.blocked_join(bits[:nq], bits[nq:], eps, precision, q_offset=0, c_offset=nq)
+                assert found == len(want) and np.array_equal(got, want), (width, precision)
+                assert secs >= 0.0
+                _, count_only, _ = oracle.blocked_join(bits[:nq], bits[nq:], eps, precision, want_pairs=False)
+                assert count_only == len(want)
+    finally:
+        oracle.blocked_join_vector_bits(native)
+
+
+def test_blocked_join_on_real_valued_data_stays_inside_the_band():
+    """Exp(40) data: the GEMM form in FP64 agrees with the difference-form checker pair for pair; in FP32 every
+    disagreement lies inside the relative 1e-3 band (count and largest error printed)."""
+    from tests import datasets
+
+    n, d = 1500, 192
+    bits = datasets.exponential(n, d, seed=5)
+    eps = datasets.epsilon_for_neighbours(bits, 20)
+    truth = oracle.self_join_f64(bits, eps)
+    got64, found64, _ = oracle.blocked_join(bits, bits, eps, 64)
+    rep64 = oracle.epsilon_band_report(bits, got64, eps, truth_pairs=truth, band=1e-9)
+    assert rep64["outside_band"] == 0, rep64
+    got32, found32, _ = oracle.blocked_join(bits, bits, eps, 32)
+    rep32 = oracle.epsilon_band_report(bits, got32, eps, truth_pairs=truth)
+    assert rep32["outside_band"] == 0, rep32
+    assert {(i, i) for i in range(n)} <= {tuple(p) for p in got32}
+    print("blocked join vs checker:", rep64, rep32)

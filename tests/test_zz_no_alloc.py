@@ -49,6 +49,39 @@ def test_no_alloc_entry_matches_the_allocating_entry_twice_in_a_row():
     assert 700 * 5 < second.pairsFound < first.pairsFound
 
 
+def test_no_alloc_entry_leaves_the_free_device_memory_unchanged_and_needs_no_library_workspace():
+    """The property the entry exists for: after the library has dropped everything it ever allocated
+    (releaseResources: resident data, workspace, pair and sort buffers), the call still works -- it uses none of
+    it -- and the free device memory reported by the driver is the same before and after further calls."""
+    import torch
+
+    import fasted_amd
+
+    lib = fasted_amd.load_findpairs()
+    bits = datasets.uniform_bytes(2000, 128, seed=9)
+    eps = datasets.epsilon_for_neighbours(bits, 10)
+    n, d = bits.shape
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    cap = 100 * n
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    lib.releaseResources()
+    torch.cuda.synchronize()
+    first = fasted_amd.self_join_device_noalloc(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap)  # looks up the array, creates its events
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        st = fasted_amd.self_join_device_noalloc(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap)
+        assert st.pairsFound == first.pairsFound > n
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    # the allocating entry on the same input, for contrast and as the reference result
+    want = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    ref = fasted_amd.self_join_device(pts.data_ptr(), n, d, d, eps, want.data_ptr(), cap, flags=1)
+    assert ref.pairsFound == first.pairsFound
+    assert np.array_equal(_row_major(pairs[: st.pairsStored].cpu().numpy()), want[: ref.pairsStored].cpu().numpy())
+
+
 def test_no_alloc_entry_refuses_what_it_cannot_do():
     import torch
 
