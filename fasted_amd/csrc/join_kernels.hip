@@ -788,26 +788,43 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                     for (int fp = 0; fp < kFragRows / 2; ++fp) asm volatile("" ::"v"(hits[fp]));
                 }
             } else if (any) {
-                // Extraction.  A round takes the first remaining hit of every lane that has one in a word of hit
-                // bits: the lanes form a mask in scalar registers, a lane's record goes behind those of the lanes
-                // before it, the wave's fill count moves on by the number of lanes.
-                auto take_round = [&](int fp, unsigned long long lanes) {
+                // Extraction.  A round takes the first remaining hit of every lane that has one among its 128
+                // elements (all four words of hit bits at once: most lanes have no hit and nearly all others
+                // exactly one, so one round is the rule): the lanes form a mask in scalar registers, a lane's
+                // record goes behind those of the lanes before it, the wave's fill count moves on by the number of
+                // lanes.  The index of a lane's first hit is a chain of vector instructions without compares
+                // (v_ffbh_u32 yields all ones for an empty word, so the minimum over the words, each with its
+                // word number in bits 5-6, is the first hit or all ones), and the two masks a round branches on --
+                // lanes with a hit, lanes with more than one -- are formed together: a branch waits for the
+                // compare that forms its mask, and one wait serves both.
+                constexpr int kWords = kFragRows / 2;
+                for (;;) {
+                    unsigned first = ~0u, total = 0u;
+#pragma unroll
+                    for (int fp = kWords - 1; fp >= 0; --fp) {
+                        unsigned lead;
+                        asm("v_ffbh_u32 %0, %1" : "=v"(lead) : "v"(hits[fp]));
+                        first = min(first, lead | (unsigned)(fp * 32));
+                        total += (unsigned)__builtin_popcount(hits[fp]);
+                    }
+                    unsigned long long lanes = __builtin_amdgcn_ballot_w64((int)first >= 0);
+                    unsigned long long again = __builtin_amdgcn_ballot_w64(total > 1u);
+                    asm volatile("" : "+s"(lanes), "+s"(again));
+                    if (lanes == 0ull) break;
                     const int count = __builtin_popcountll(lanes) << (mirror ? 1 : 0);
                     if (staged + count > kWaveStagePairs) flush_wave();
-                    unsigned& w = hits[fp];
-                    if (w != 0u) {
-                        const int e = __builtin_clz(w);  // element number inside the pair of block rows
-                        w &= ~(0x80000000u >> e);
-                        const int q = qLane + fp * 32 + (e >> 4) * 16 + (e & 3);
-                        const int c = cLane + ((e >> 2) & 3) * 16;
+                    if ((int)first >= 0) {
+                        // element `first` of the lane: block row first / 16, block column (first / 4) % 4, row first % 4
+                        const int q = qLane + (int)((first & ~15u) + (first & 3u));
+                        const int c = cLane + (int)((first & 12u) << 2);
                         const unsigned before = __builtin_amdgcn_mbcnt_hi(
                             (unsigned)(lanes >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)lanes, 0u));
                         const unsigned at = (unsigned)staged + (mirror ? 2u * before : before);
                         // written as an instruction: for an ordinary LDS store the compiler first waits until
                         // this wave's global->LDS transfers of the next tile have landed
-                        auto put = [&](unsigned idx, int first, int second) {
+                        auto put = [&](unsigned idx, int a0, int a1) {
                             const unsigned long long rec =
-                                (unsigned long long)(unsigned)first | ((unsigned long long)(unsigned)second << 32);
+                                (unsigned long long)(unsigned)a0 | ((unsigned long long)(unsigned)a1 << 32);
                             asm volatile("ds_write_b64 %0, %1" ::"v"(ldsBase + (unsigned)kLdsStage +
                                                                      ((unsigned)wave * kWaveStagePairs + idx) * 8u),
                                          "v"(rec)
@@ -817,28 +834,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                         if (mirror) put(at + 1, c, q);
                     }
                     staged += count;
-                };
-                // The four words' masks are formed together, and again together after every word has had a round
-                // (a branch on a mask waits for the compare that forms it: one at a time, that wait is paid per
-                // word and round; most lanes have one hit at most, so the second set of masks is usually empty).
-                unsigned long long lanes[kFragRows / 2];
-                auto form_masks = [&]() {
+                    if (again == 0ull) break;
+                    // some lane has another hit: every lane drops the one it has just written
 #pragma unroll
-                    for (int fp = 0; fp < kFragRows / 2; ++fp) lanes[fp] = __builtin_amdgcn_ballot_w64(hits[fp] != 0u);
-#pragma unroll
-                    for (int fp = 0; fp < kFragRows / 2; ++fp) asm volatile("" : "+s"(lanes[fp]));
-                };
-                form_masks();
-#pragma unroll
-                for (int fp = 0; fp < kFragRows / 2; ++fp)
-                    if (lanes[fp] != 0ull) take_round(fp, lanes[fp]);
-                form_masks();
-#pragma unroll
-                for (int fp = 0; fp < kFragRows / 2; ++fp)
-                    while (lanes[fp] != 0ull) {
-                        take_round(fp, lanes[fp]);
-                        lanes[fp] = __builtin_amdgcn_ballot_w64(hits[fp] != 0u);
-                    }
+                    for (int fp = 0; fp < kWords; ++fp)
+                        if ((first >> 5) == (unsigned)fp) hits[fp] &= ~(0x80000000u >> (first & 31u));
+                }
             }
         } else {
             // keep the accumulators observable without spending instructions on them
