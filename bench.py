@@ -363,7 +363,8 @@ def main():
                    "library_path": fp.library_path(), "peak_used_tflops": PEAK_FP16_TFLOPS, "clocks": clocks.summary()},
         "roofline": {"bound": "mfma", "kernel": "join_kernel", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
-                     "traffic": traffic, "traffic_detail": traffic_detail},
+                     "traffic": traffic, "traffic_detail": traffic_detail,
+                     "traffic_source": (traffic_detail or {}).get("source")},
     }
     # Parity is part of the measurement: a line whose pair set fails the check (a sampled pair outside the
     # relative 1e-3 band around epsilon, a pair buffer that overflowed so that nothing could be checked, a

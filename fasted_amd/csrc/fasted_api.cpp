@@ -1080,6 +1080,8 @@ int fasted_self_join_device_noalloc(const void* d_points, long long n, int d, lo
             throw std::invalid_argument("fasted_self_join_device_noalloc cannot sort: the sort allocates device memory");
         if (flags & FASTED_SKIP_SUMS)
             throw std::invalid_argument("fasted_self_join_device_noalloc computes the squared norms itself");
+        validate_epsilon(epsilon);
+        validate_shape(n, d, ld);
         DeviceScratch& ds = device_scratch();
         float* const norms = reinterpret_cast<float*>(ds.base + kNoAllocCounterBytes);
         const JoinScratch js{reinterpret_cast<unsigned long long*>(ds.base), norms, norms + kNoAllocMaxPoints, ds.ev};
@@ -1146,6 +1148,7 @@ int fasted_self_join(const uint16_t* points, long long n, int d, double epsilon,
         if (!points) throw std::invalid_argument("points pointer is null");
         if (cap > 0 && !out) throw std::invalid_argument("output buffer is null");
         if (n < 1 || d < 1) throw std::invalid_argument("empty dataset");
+        validate_epsilon(epsilon);
         const int dPad = round_up(d, fasted::kSlabK);
         validate_shape(n, d, dPad);
         void* dPoints = nullptr;

@@ -150,6 +150,18 @@ def test_raw_entry_rejects_bad_arguments_without_touching_a_gpu(lib):
         assert rc != 0 and lib.fasted_last_error()
     assert lib.fasted_self_join_blocked(ctypes.addressof(buf), 10, 8, 0.1, 0, None, 0, None, None) != 0
     assert b"block" in lib.fasted_last_error()
+    # a NaN epsilon is refused by every entry that takes one, before any device call (the reference's comparison
+    # with NaN is false for every pair, source/warpMma.cuh:257; here it would poison the accumulator start values)
+    nan = float("nan")
+    assert lib.fasted_self_join(ctypes.addressof(buf), 4, 8, nan, None, 0, ctypes.byref(found), ctypes.byref(stored)) != 0
+    assert b"NaN" in lib.fasted_last_error()
+    assert lib.fasted_self_join_device(ctypes.addressof(buf), 1, 64, 64, nan, None, None, 0, 0, None, ctypes.byref(st)) != 0
+    assert b"NaN" in lib.fasted_last_error()
+    assert lib.fasted_self_join_device_noalloc(ctypes.addressof(buf), 1, 64, 64, nan, None, 0, 0, None, ctypes.byref(st)) != 0
+    assert lib.fasted_join_device(ctypes.addressof(buf), 1, 64, ctypes.addressof(buf), 1, 64, 64, nan, None, None, None, 0,
+                                  0, None, ctypes.byref(st)) != 0
+    assert lib.fasted_self_join_blocked(ctypes.addressof(buf), 4, 8, nan, 256, None, 0, None, None) != 0
+    assert b"NaN" in lib.fasted_last_error()
     assert lib.fasted_pair_distances_device(None, 1, 64, None, 1, 64, 64, None, 0, None, None) != 0
 
 
