@@ -295,12 +295,22 @@ __device__ __forceinline__ void static_for(F&& f) {
 // that matters at such sizes and keeps one set of addresses.
 // kOneSlab: D <= 64, a tile is one slab.  No barrier inside such a tile could publish the next tile's coordinates, so
 // the mailbox that carries them runs one tile further ahead there (two slots).
-template <bool kEpilogue, bool kTall, int kTileRows, bool kOneSlab>
+// kBitsInLastSlab: the hit bits of a tile are gathered between the MFMAs of its last slab instead of behind the
+// k-loop (tiles of up to 16 slabs; see slab_step).
+template <bool kEpilogue, bool kTall, int kTileRows, bool kOneSlab, bool kBitsInLastSlab = false>
 __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
+    static_assert(!kBitsInLastSlab || kEpilogue, "hit bits are gathered only when there is an epilogue");
     static_assert(kTileRows == 256 || kTileRows == 128, "tile rows");
     constexpr int kWaveRows = kTileRows / 2;    // rows of a wave's output sub-tile (2 x 4 waves)
     constexpr int kFragRows = kWaveRows / 16;   // its rows of 16x16 blocks
     constexpr int kHalfRows = kFragRows / 2;    // a k-step goes through them in two halves
+    // Tiles of up to 16 slabs gather their hit bits between the MFMAs of their last slab (see slab_step).  Against
+    // screening the accumulators behind the k-loop, on workloads with neighbours to report: +9 % at 200k x 64 and
+    // +6.6 % at 100k x 128 (64 neighbours), +2.1 % at 2M x 384 (1000), +3 / +2 / +1 % at D = 256 / 512 / 1024 (100);
+    // when no tile has a hit it costs instead: -2 % at D = 64, -0.6 % at 256, -0.2 % at 1024.  Longer tiles keep
+    // the screening, which is the cheaper of the two when hardly any tile has a hit (0.1 - 0.3 % at D = 4096 with 16
+    // neighbours); a run-time choice between the two inside one kernel made the register allocator spill.
+    constexpr bool kFusedBits = kBitsInLastSlab;
     __shared__ __align__(16) unsigned char lds[kLdsBytes];
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);  // wave-uniform, lives in an SGPR
     const int wr = wave >> 2, wc = wave & 3;
@@ -514,6 +524,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // set between the MFMAs of the tile's first k-step, one row of blocks ahead of the MFMAs that need it
         // (a wave's vector instructions between its own MFMAs cost far less than on their own).
         floatx4 acc[kFragRows][kFragCols];
+        // Per-lane hit bits of the 4 pairs of block rows: element e = (fi & 1) * 16 + fj * 4 + r of the pair
+        // fi / 2 is bit 31 - e.
+        unsigned hits[kFragRows / 2];
         float hc[kFragCols];
         const float* sQw;
         {
@@ -545,11 +558,81 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         // the first k-step, four at the start of each of its halves: early, so that an L2 miss has the
         // whole second k-step to land before the slab's barrier (one transfer pinned in front of every 4 MFMAs
         // instead measured 1-3 % slower on the 1M x 4096 workload).
-        auto slab_step = [&](auto firstc, int stg, bool prefetch, const char* pA, const char* pB,
+        auto slab_step = [&](auto modec, int stg, bool prefetch, const char* pA, const char* pB,
                              const unsigned (&oA)[4], const unsigned (&oB)[4]) {
-            constexpr bool first = decltype(firstc)::value;  // the tile's first slab also sets the accumulators
+            constexpr int mode = decltype(modec)::value;
+            constexpr bool first = mode == 1;     // the tile's first slab also sets the accumulators
+            constexpr bool withBits = mode == 2;  // the tile's last slab also gathers the hit bits
             const unsigned char* const buf = lds + stg * kStageBytes;
             half8 aLo[kHalfRows], aHi[kHalfRows], b[2][kFragCols];
+
+            if constexpr (withBits) {
+                // The tile's last slab goes through the rows of blocks one after the other like the first, both
+                // k-steps of a row together: after its 8 MFMAs a row of blocks is final, and the sign bits of its
+                // 16 elements per lane (set = no hit) are shifted into the lane's hit words between the 8 MFMAs of
+                // the row after it, two vector instructions behind every MFMA, where they cost next to nothing
+                // -- instead of a screening pass over all accumulators and a conditional pass over the rows with
+                // a hit behind the k-loop, where nothing hides them.  Only the last row's 16 shifts are exposed.
+                // (Both k-steps visit the candidate blocks in ascending order, so that the blocks of a row become
+                // final in the order in which their bits are gathered.)
+                half8 a[2][2];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    a[0][ks] = fragment(buf + aOff[ks]);
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj) b[ks][fj] = fragment(buf + bOff[ks] + fj * 16 * kRowBytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                unsigned m = ~0u;
+                auto gather_row = [&](int fi) {
+#pragma unroll
+                    for (int fj = 0; fj < kFragCols; ++fj)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const float v = acc[fi][fj][r];
+                            m = __builtin_amdgcn_alignbit(m, __float_as_uint(v), 31);
+                        }
+                    // (an anchor: without it the shifts are sunk to where the hit words are used, behind the k-loop)
+                    asm volatile("" : "+v"(m));
+                    if (fi & 1) {
+                        hits[fi >> 1] = kNoHits ? 0u : ~m;
+                        m = ~0u;
+                    }
+                };
+                static_for<0, kFragRows>([&](auto fic) {
+                    constexpr int fi = decltype(fic)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (fi < 4) {
+                        if (prefetch) {
+                            issue_load(std::integral_constant<int, 2 * fi>{}, pA, pB, oA, oB, stg ^ 1);
+                            issue_load(std::integral_constant<int, 2 * fi + 1>{}, pA, pB, oA, oB, stg ^ 1);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (fi + 1 < kFragRows) {
+                        a[(fi + 1) & 1][0] = fragment(buf + aOff[0] + (fi + 1) * 16 * kRowBytes);
+                        a[(fi + 1) & 1][1] = fragment(buf + aOff[1] + (fi + 1) * 16 * kRowBytes);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int fj = 0; fj < kFragCols; ++fj)
+                            acc[fi][fj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[fi & 1][ks], b[ks][fj], acc[fi][fj], 0, 0, 0);
+                    if constexpr (fi >= 1) {
+                        gather_row(fi - 1);
+                        // the order asked of the scheduler: the fragment reads, then MFMA, 2 shifts, MFMA, 2 shifts ...
+                        if constexpr (fi + 1 < kFragRows) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                        }
+                    }
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                gather_row(kFragRows - 1);
+                return;
+            }
 
             if constexpr (first) {
                 // The tile's first slab goes through the rows of blocks one after the other, both k-steps of a
@@ -656,8 +739,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             }
         };
 
-        constexpr std::integral_constant<bool, true> kFirstSlab{};
-        constexpr std::integral_constant<bool, false> kLaterSlab{};
+        constexpr std::integral_constant<int, 1> kFirstSlab{};
+        constexpr std::integral_constant<int, 0> kLaterSlab{};
+        constexpr std::integral_constant<int, kFusedBits ? 2 : 0> kLastSlab{};
         if (!kOneSlab && p.nSlabs > 1) {  // (the run-time test is always true here; the register allocator does better with it)
             slab_step(kFirstSlab, stage, true, gA + kRowBytes, gB + kRowBytes, offA, offB);
             stage ^= 1;
@@ -686,7 +770,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
 #pragma unroll
             for (int fi = 1; fi < kFragRows; ++fi) init_row(fi);
         }
-        slab_step(kLaterSlab, stage, more, gA, gB, offA, offB);
+        slab_step(kLastSlab, stage, more, gA, gB, offA, offB);
         stage ^= 1;
 
         if (kEpilogue) {
@@ -708,11 +792,14 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             const bool edge = nonFinite || diagonal || rowBase + kTileRows > p.nQ || colBase + kTile > p.nC;
             const bool mirror = p.symmetric && tr != tc;  // a tile above the diagonal also stands for its mirror image
 
-            // Per-lane hit bits of the 4 pairs of block rows: element e = (fi & 1) * 16 + fj * 4 + r of the pair
-            // fi / 2 is bit 31 - e.
-            unsigned hits[kFragRows / 2];
             bool any;
-            if (!edge) {
+            if (kFusedBits && !edge) {
+                // the hit bits came out of the last slab: is there one in the wave at all?
+                unsigned some = hits[0];
+#pragma unroll
+                for (int fp = 1; fp < kFragRows / 2; ++fp) some |= hits[fp];
+                any = __builtin_amdgcn_ballot_w64(some != 0u) != 0ull;
+            } else if (!edge) {
                 // Screening, about 1/2 vector instruction per element: the maximum of the lane's 128 elements,
                 // formed per row of blocks; a wave in which no lane has a hit is done.
                 float rowBest[kFragRows];
@@ -992,24 +1079,38 @@ hipError_t launch_join_grid(JoinParams p, bool rows128, bool tall, bool epilogue
     if (grid == 0) grid = 1;
     const dim3 g(grid), b(kThreads);
     const bool oneSlab = p.nSlabs == 1;
-    const int variant = (oneSlab ? 8 : 0) | (epilogue ? 4 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
-    switch (variant) {
-        case 15: join_kernel<true, true, 128, true><<<g, b, 0, stream>>>(p); break;
-        case 14: join_kernel<true, true, 256, true><<<g, b, 0, stream>>>(p); break;
-        case 13: join_kernel<true, false, 128, true><<<g, b, 0, stream>>>(p); break;
-        case 12: join_kernel<true, false, 256, true><<<g, b, 0, stream>>>(p); break;
-        case 11: join_kernel<false, true, 128, true><<<g, b, 0, stream>>>(p); break;
-        case 10: join_kernel<false, true, 256, true><<<g, b, 0, stream>>>(p); break;
-        case 9: join_kernel<false, false, 128, true><<<g, b, 0, stream>>>(p); break;
-        case 8: join_kernel<false, false, 256, true><<<g, b, 0, stream>>>(p); break;
-        case 7: join_kernel<true, true, 128, false><<<g, b, 0, stream>>>(p); break;
-        case 6: join_kernel<true, true, 256, false><<<g, b, 0, stream>>>(p); break;
-        case 5: join_kernel<true, false, 128, false><<<g, b, 0, stream>>>(p); break;
-        case 4: join_kernel<true, false, 256, false><<<g, b, 0, stream>>>(p); break;
-        case 3: join_kernel<false, true, 128, false><<<g, b, 0, stream>>>(p); break;
-        case 2: join_kernel<false, true, 256, false><<<g, b, 0, stream>>>(p); break;
-        case 1: join_kernel<false, false, 128, false><<<g, b, 0, stream>>>(p); break;
-        default: join_kernel<false, false, 256, false><<<g, b, 0, stream>>>(p); break;
+    // Tiles of up to 16 slabs gather their hit bits in their last slab; longer ones screen behind the k-loop.
+    const bool bitsInLastSlab = epilogue && p.nSlabs <= 16;
+    const int variant = (oneSlab ? 8 : 0) | (tall ? 2 : 0) | (rows128 ? 1 : 0);
+    if (bitsInLastSlab) {
+        switch (variant) {
+            case 11: join_kernel<true, true, 128, true, true><<<g, b, 0, stream>>>(p); break;
+            case 10: join_kernel<true, true, 256, true, true><<<g, b, 0, stream>>>(p); break;
+            case 9: join_kernel<true, false, 128, true, true><<<g, b, 0, stream>>>(p); break;
+            case 8: join_kernel<true, false, 256, true, true><<<g, b, 0, stream>>>(p); break;
+            case 3: join_kernel<true, true, 128, false, true><<<g, b, 0, stream>>>(p); break;
+            case 2: join_kernel<true, true, 256, false, true><<<g, b, 0, stream>>>(p); break;
+            case 1: join_kernel<true, false, 128, false, true><<<g, b, 0, stream>>>(p); break;
+            default: join_kernel<true, false, 256, false, true><<<g, b, 0, stream>>>(p); break;
+        }
+    } else if (epilogue) {  // more than 16 slabs
+        switch (variant) {
+            case 3: join_kernel<true, true, 128, false><<<g, b, 0, stream>>>(p); break;
+            case 2: join_kernel<true, true, 256, false><<<g, b, 0, stream>>>(p); break;
+            case 1: join_kernel<true, false, 128, false><<<g, b, 0, stream>>>(p); break;
+            default: join_kernel<true, false, 256, false><<<g, b, 0, stream>>>(p); break;
+        }
+    } else {
+        switch (variant) {
+            case 11: join_kernel<false, true, 128, true><<<g, b, 0, stream>>>(p); break;
+            case 10: join_kernel<false, true, 256, true><<<g, b, 0, stream>>>(p); break;
+            case 9: join_kernel<false, false, 128, true><<<g, b, 0, stream>>>(p); break;
+            case 8: join_kernel<false, false, 256, true><<<g, b, 0, stream>>>(p); break;
+            case 3: join_kernel<false, true, 128, false><<<g, b, 0, stream>>>(p); break;
+            case 2: join_kernel<false, true, 256, false><<<g, b, 0, stream>>>(p); break;
+            case 1: join_kernel<false, false, 128, false><<<g, b, 0, stream>>>(p); break;
+            default: join_kernel<false, false, 256, false><<<g, b, 0, stream>>>(p); break;
+        }
     }
     return hipGetLastError();
 }

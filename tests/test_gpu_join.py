@@ -75,10 +75,12 @@ def test_sum_squared_closed_form_integer_rows(fasted):
     assert np.allclose(got, expect, rtol=64 * 2.0 ** -24)
 
 
-@pytest.mark.parametrize("n,d", [(256, 64), (512, 128), (300, 64), (1025, 192), (2048, 1024)])
+@pytest.mark.parametrize("n,d", [(256, 64), (512, 128), (300, 64), (1025, 192), (2048, 1024), (700, 1536), (1300, 2048)])
 def test_integer_points_exact_pair_set(fasted, n, d):
     """Integer coordinates make every dot product exact, so the pair set must equal the FP64
-    join bit for bit (epsilon^2 sits between two integers: no pair is near the threshold)."""
+    join bit for bit (epsilon^2 sits between two integers: no pair is near the threshold).  Tiles of up to 16
+    slabs (D <= 1024) gather their hit bits in their last slab, longer ones screen their accumulators behind the
+    k-loop: both kinds are here."""
     bits = datasets.small_integers(n, d, high=3, seed=7 * n + d)
     x = bits.view(np.float16).astype(np.float64)
     d2 = ((x[:64, None, :] - x[None, :64, :]) ** 2).sum(-1)
