@@ -120,6 +120,22 @@ def test_native_epsilon_search_matches_the_python_procedure(lib):
     lib.releaseResources()
 
 
+@pytest.mark.parametrize("n,d", [(3000, 320), (20000, 192)])
+def test_count_only_probe_equals_the_full_join_count(lib, n, d):
+    """The count-only probe computes the tiles on and above the diagonal only and doubles what it finds off the
+    diagonal; a storing reRun computes the whole matrix.  The two counts must be equal at every epsilon (144 tiles
+    one per workgroup, and 6241 tiles through the queues in the tall order)."""
+    import fasted_amd
+
+    assert lib.fasted_load_exponential_dataset(n, d, 40.0, 10.0) == 0
+    eps, sel, _ = fasted_amd.find_epsilon_sampled(24.0, sample_rows=2000)
+    for e in (eps, 0.8 * eps, 1e-4):
+        found, secs = fasted_amd.count_pairs(e)
+        r = lib.reRun(e, False)
+        assert found == r.pairsFound >= n and secs > 0, e
+    lib.releaseResources()
+
+
 def test_pairs_can_stay_on_the_device(lib):
     """With the download switched off a run that does not save reports the same Results and leaves the sorted pairs
     in the library's device buffer, where fasted_last_pairs_device finds them; a saving run still writes its file."""
