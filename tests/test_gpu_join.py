@@ -478,7 +478,8 @@ def test_both_tile_heights_give_the_exact_pair_set(fasted, n, d, monkeypatch):
 def test_small_joins_time_themselves_with_the_device_clock(fasted):
     """Joins of at most 512 tiles are timed by clock readings of the kernels themselves instead of events: the two
     times must be positive, add up to less than the wall time of the call, and agree with the event-timed figure
-    of the same kernel on a matrix just large enough to be timed with events (same D, per-tile time within 2x)."""
+    of the same kernel on a matrix just large enough to be timed with events (same D, per-tile time within 3x: a
+    check of the unit of the clock, not of the speed)."""
     import time
 
     import torch
@@ -506,4 +507,4 @@ def test_small_joins_time_themselves_with_the_device_clock(fasted):
     tb = min(fasted.self_join_device(ptsb.data_ptr(), 6000, d, d, eps, pb.data_ptr(), pb.shape[0], flags=0).joinMs
              for _ in range(10))
     per_tile_small, per_tile_big = best / 1.0, tb / 3.0  # one round of the 256 workgroups against three
-    assert 0.5 < per_tile_small / per_tile_big < 2.0, (best, tb)
+    assert 1.0 / 3.0 < per_tile_small / per_tile_big < 3.0, (best, tb)
