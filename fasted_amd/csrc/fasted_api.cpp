@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <climits>
@@ -82,10 +83,17 @@ struct Workspace {
     }
 
     void ensure(size_t n) {
-        if (!counters) HIP_CHECK(hipMalloc(&counters, fasted::counter_words() * sizeof(unsigned long long)));
         if (!hostCount) {
             HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocDefault));
             HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&hostCountDev), hostCount, 0));
+        }
+        if (!counters) {
+            // all zero (the non-finite flag is compared with join numbers, which start at 1), except for the word
+            // that tells the join kernel where to report the pair count and its clock readings
+            const size_t bytes = fasted::counter_words() * sizeof(unsigned long long);
+            HIP_CHECK(hipMalloc(&counters, bytes));
+            HIP_CHECK(hipMemset(counters, 0, bytes));
+            HIP_CHECK(hipMemcpy(counters + fasted::host_words_slot(), &hostCountDev, sizeof hostCountDev, hipMemcpyHostToDevice));
         }
         for (auto& e : ev)
             if (!e) HIP_CHECK(hipEventCreate(&e));
@@ -251,8 +259,8 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     const unsigned long long epoch = ++g_epoch;
     // Timing.  Three event records cost a call about 10 us, a third of a join of a few thousand points, so a
     // join of at most two tiles per compute unit is timed by the kernels themselves instead: the first norm
-    // kernel and the join kernel note the device's constant-rate clock when they start, and so does the
-    // one-thread kernel behind the join that hands the pair count to the host.  Larger joins, and the entry
+    // kernel and the join kernel note the device's constant-rate clock when they start, and the join kernel's
+    // last workgroup when it hands the pair count to the host.  Larger joins, and the entry
     // that owns no pinned memory, are timed with events on the stream as the reference is
     // (source/findPairs.cuh:625-639,695-697,728-736).
     const bool stamped = !fixed && fasted::tile_count(q.n, c.n) <= 512;
@@ -286,6 +294,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     jl.pairs = dPairs;
     jl.cap = cap;
     jl.epilogue = !(flags & FASTED_NO_EPILOGUE);
+    if (!fixed) static_cast<volatile unsigned long long*>(g_ws.hostCount)[3] = 0;  // the kernel's report turns it non-zero
     HIP_CHECK(fasted::launch_join(jl, stream));
     if (events) HIP_CHECK(hipEventRecord(t.ev[2], stream));
     // c[0] = pairs found; every slot below the capacity received exactly one pair, the rest were
@@ -295,11 +304,21 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
         HIP_CHECK(hipStreamSynchronize(stream));
         HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
     } else {
-        // the count (and the kernels' clock readings) travel behind the join kernel into pinned memory, written
-        // by a one-thread kernel: one wait for kernels and count
-        HIP_CHECK(fasted::launch_publish_count(counters, g_ws.hostCountDev, stream));
-        HIP_CHECK(hipStreamSynchronize(stream));
-        cnt[0] = static_cast<volatile unsigned long long*>(g_ws.hostCount)[0];
+        // The join kernel's last workgroup writes the count (and the kernels' clock readings) into pinned memory:
+        // no launch or copy command behind the join.  A small join is over when that report is there -- every
+        // workgroup has released its stores at system scope before it was counted -- and the few microseconds
+        // until the stream itself reports idle, a fifth of such a call, are not waited for.  (A kernel that never
+        // reports, because it failed, falls through to the stream's own wait, which returns the error.)
+        volatile unsigned long long* const w = g_ws.hostCount;
+        bool reported = false;
+        if (stamped) {
+            const auto t0 = std::chrono::steady_clock::now();
+            for (unsigned spins = 1; !(reported = w[3] != 0); ++spins)
+                if ((spins & 1023u) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) break;
+            std::atomic_thread_fence(std::memory_order_acquire);
+        }
+        if (!reported) HIP_CHECK(hipStreamSynchronize(stream));
+        cnt[0] = w[0];
     }
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);

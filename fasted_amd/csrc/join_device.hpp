@@ -12,14 +12,21 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Counter block of one join: word 0 = pairs found, word 1 = non-finite flag, words 2 and 3 = clock readings,
-// then the 8 queue heads, each on its own 128-byte line.
+// Counter block of one join: word 0 = pairs found, word 1 = non-finite flag, word 2 = a clock reading, word 3 =
+// workgroups of the join kernel that have signed off; then the 8 queue heads, each on its own 128-byte line; then,
+// on a line of its own again (it is read by every workgroup while the first line is busy with atomics), where the
+// join kernel reports to the host.
 constexpr int kCounterFound = 0;
 constexpr int kCounterNonFinite = 1;  // == the join's epoch: some point of the join has a non-finite squared norm
 constexpr int kCounterStampNorms = 2;  // the device's constant-rate clock when the join's first norm kernel started
-constexpr int kCounterStampJoin = 3;   // ... when the join kernel started
+constexpr int kCounterDone = 3;        // workgroups of the join kernel that are through (the last one reports to the host)
 constexpr int kQueueBase = 16, kQueueStride = 16;
-constexpr int kCounterWords = kQueueBase + kQueues * kQueueStride;
+// Set once by the owner of the block and never cleared by a kernel: the address (as the device sees it) of 4 words
+// of pinned host memory, or 0: [0] pairs found, [1]-[3] clock readings (norms started, join kernel started, join
+// kernel through).  It sits here and not among the kernel's arguments because the tile loop has no scalar
+// registers to spare.
+constexpr int kCounterHostWords = kQueueBase + kQueues * kQueueStride;
+constexpr int kCounterWords = kCounterHostWords + 16;
 
 struct JoinParams {
     const u32x4* ptsQ;  // query rows

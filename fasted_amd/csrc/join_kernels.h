@@ -22,7 +22,13 @@ struct JoinLaunch {
     int dPad;                    // K extent, multiple of kSlabK
     const float* halfQ;          // per query point: eps^2/4 - s/2 (s = squared norm), see launch_sum_squared
     const float* halfC;          // ... per candidate point
-    unsigned long long* counters;  // counter_words() words: [0] pairs found, [1] non-finite flag, then the queue heads
+    unsigned long long* counters;  // counter_words() words: [0] pairs found, [1] non-finite flag, ..., then the queue
+                                   // heads.  Word host_words_slot() is the owner's: the device-side address of 4
+                                   // words of pinned host memory, or 0.  If set, the join kernel's last workgroup
+                                   // writes [0] = pairs found and the device's constant-rate clock [1] when the
+                                   // join's first norm kernel started and [3] (never 0) when it was through itself,
+                                   // its first workgroup [2] when it started; every pair record of the join is in
+                                   // memory when [3] appears.  The kernels of this file never clear that word.
     unsigned long long epoch = 1;  // number of the join: what the norm kernels of THIS join write into the
                                    // non-finite flag (a flag left by an earlier join is not seen)
     void* pairs;                 // FastedPair[cap]
@@ -35,6 +41,7 @@ struct JoinLaunch {
 unsigned long long raster_count(long long nQ, long long nC, bool upperOnly = false);
 int raster_coord(unsigned long long idx, long long nQ, long long nC, bool upperOnly, int* row, int* col);
 int counter_words();
+int host_words_slot();
 unsigned long long tile_count(long long nQ, long long nC);  // 256x256 tiles the kernel processes
 // Slot (0..7) of 16-byte chunk `chunk` of slab row `row` in LDS (host mirror of the device swizzle).
 int lds_chunk_slot(int row, int chunk);
@@ -55,9 +62,6 @@ hipError_t launch_padding_check(const void* points, long long ld, int n, int d, 
                                 hipStream_t stream);
 // Clears the queue heads and, unless keepFound, the pair counter (word 0 of `counters`).
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream);
-// hostWords (pinned host memory, device-visible address) [0] = the pair counter, [1], [2] = the constant-rate clock
-// at the start of the join's first norm kernel and of the join kernel, [3] = now; written by a one-thread kernel.
-hipError_t launch_publish_count(const unsigned long long* counters, unsigned long long* hostWords, hipStream_t stream);
 // pairs[first, last): QueryPoint += qOffset, CandidatePoint += cOffset.
 hipError_t launch_offset_pairs(void* pairs, unsigned long long first, unsigned long long last, int qOffset, int cOffset,
                                hipStream_t stream);

@@ -136,7 +136,7 @@ __device__ __forceinline__ void reset_for_join(unsigned long long* __restrict__ 
     if (blockIdx.x != 0) return;
     const int t = threadIdx.x;
     if (t == 0) counters[kCounterStampNorms] = wall_clock64();  // the timed region of a small join starts here
-    if (t < kCounterWords && t != kCounterNonFinite && t != kCounterStampNorms && t != kCounterStampJoin) counters[t] = 0ull;
+    if (t < kCounterWords && t != kCounterNonFinite && t != kCounterStampNorms && t != kCounterHostWords) counters[t] = 0ull;
 }
 
 __global__ void __launch_bounds__(256) sum_squared_kernel(const u32x4* __restrict__ pts, long long ld16, int n,
@@ -218,20 +218,9 @@ __global__ void __launch_bounds__(256) padding_check_kernel(const unsigned short
 // of the join that raised it.  (A join that computes its norms first needs no launch of this: the norm kernel's
 // first workgroup does the clearing.)
 __global__ void reset_counters_kernel(unsigned long long* c, int keepFound) {
-    if (threadIdx.x < kCounterWords && threadIdx.x != kCounterNonFinite && !(keepFound && threadIdx.x == kCounterFound))
+    if (threadIdx.x < kCounterWords && threadIdx.x != kCounterNonFinite && threadIdx.x != kCounterHostWords &&
+        !(keepFound && threadIdx.x == kCounterFound))
         c[threadIdx.x] = 0ull;
-}
-
-// Copies the pair counter and the clock readings of the norm and join kernels into pinned host memory that the
-// device can write, and adds its own reading: it starts when the join kernel is over.  (A one-thread kernel behind
-// the join is no slower than a copy command of a few bytes, and its clock reading replaces an event.)
-__global__ void publish_count_kernel(const unsigned long long* __restrict__ counters, unsigned long long* hostWords) {
-    const unsigned long long now = wall_clock64();
-    hostWords[0] = counters[kCounterFound];
-    hostWords[1] = counters[kCounterStampNorms];
-    hostWords[2] = counters[kCounterStampJoin];
-    hostWords[3] = now;
-    __threadfence_system();
 }
 
 // Adds the first row of the query block and of the candidate block to the pairs [first, last) that a
@@ -334,7 +323,34 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     unsigned* const sNext = reinterpret_cast<unsigned*>(lds + kLdsNext);  // two slots of [0] row, [1] col
     const int2* const sStage = reinterpret_cast<const int2*>(lds + kLdsStage) + wave * kWaveStagePairs;  // this wave's region
 
-    if (blockIdx.x == 0 && threadIdx.x == 0) p.counters[kCounterStampJoin] = wall_clock64();  // (timing of small joins)
+    // (timing of small joins: the first workgroup notes when the kernel started, straight into the host's words)
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        unsigned long long* const hostWords = reinterpret_cast<unsigned long long*>(p.counters[kCounterHostWords]);
+        if (hostWords) __hip_atomic_store(&hostWords[2], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+
+    // Every workgroup signs off when it has nothing left to do, and the one that signs off last hands the pair
+    // count and the clock readings to the host (pinned memory that the device writes): no launch and no copy
+    // command behind the join for that, and the host may take a small join for finished when word 3 turns
+    // non-zero, without waiting for the stream.  So a workgroup is counted only when its pair records have
+    // arrived in memory: they are written through (store_pair), each wave waits for its own, the barrier
+    // collects the waves.  (A release fence per workgroup would do the same by writing the whole L2 back, once
+    // per workgroup: measured, 2 us on a join of 13 us and 11 us on one of 190 us.)  A workgroup's additions to the
+    // pair counter are over by then as well -- their old values have come back and been used -- so the last to
+    // sign off reads the final count.
+    auto sign_off = [&]() {
+        unsigned long long* const hostWords = reinterpret_cast<unsigned long long*>(p.counters[kCounterHostWords]);
+        if (!hostWords) return;
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        __syncthreads();
+        if (threadIdx.x != 0) return;
+        if (atomicAdd(&p.counters[kCounterDone], 1ull) + 1 != gridDim.x) return;
+        __hip_atomic_store(&hostWords[0], atomicAdd(&p.counters[kCounterFound], 0ull), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(&hostWords[1], p.counters[kCounterStampNorms], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // both are on their way before the word that the host watches
+        __hip_atomic_store(&hostWords[3], wall_clock64() | 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    };
 
     // set by the kernel that formed this join's per-point halves: some point has a non-finite squared norm
     const bool nonFinite = p.counters[kCounterNonFinite] == p.epoch;
@@ -379,6 +395,14 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // reservation on the global counter (same-address atomics serialise at about 12 ns each: one per pair,
     // or per wave and tile, is what would bound output-heavy joins) and coalesced 8-byte stores.
     int staged = 0;
+    // Pair records are written through to memory (a store at system scope) instead of staying dirty in the L2 of
+    // the XCD until the kernel ends: the host may take a small join for finished as soon as the last workgroup
+    // has reported, and a record is written once and not read again by this kernel.
+    auto store_pair = [&](unsigned long long slot, int2 rec) {
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(p.pairs + slot),
+                           (unsigned long long)(unsigned)rec.x | ((unsigned long long)(unsigned)rec.y << 32),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    };
     auto flush_wave = [&]() {
         const int ln = lane_now();
         unsigned long long base = 0;
@@ -387,7 +411,7 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
                __builtin_amdgcn_readfirstlane((unsigned)base);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staged records are in LDS
         for (int i = ln; i < staged; i += 64)
-            if (base + i < p.cap) p.pairs[base + i] = sStage[i];  // past the capacity: counted, not stored
+            if (base + i < p.cap) store_pair(base + i, sStage[i]);  // past the capacity: counted, not stored
         staged = 0;
     };
 
@@ -482,7 +506,10 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     __syncthreads();
     unsigned tr = __builtin_amdgcn_readfirstlane(sNext[0]);
     unsigned tc = __builtin_amdgcn_readfirstlane(sNext[1]);
-    if (tr == kNoTile) return;
+    if (tr == kNoTile) {
+        sign_off();
+        return;
+    }
 
     unsigned offA[4], offB[4];
     tile_offsets((int)tr * kTileRows, (int)tc * kTile, offA, offB, true);
@@ -958,13 +985,15 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
             if (w < wave) before += left;
             total += left;
         }
-        if (total == 0) return;
-        if (wave == 0 && ln == 0) *sBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)total);
-        __syncthreads();
-        const unsigned long long base = *sBase + before;
-        for (int i = ln; i < staged; i += 64)
-            if (base + i < p.cap) p.pairs[base + i] = sStage[i];
+        if (total != 0) {
+            if (wave == 0 && ln == 0) *sBase = atomicAdd(&p.counters[kCounterFound], (unsigned long long)total);
+            __syncthreads();
+            const unsigned long long base = *sBase + before;
+            for (int i = ln; i < staged; i += 64)
+                if (base + i < p.cap) store_pair(base + i, sStage[i]);
+        }
     }
+    sign_off();
 }
 
 }  // namespace
@@ -988,6 +1017,7 @@ int raster_coord(unsigned long long idx, long long nQ, long long nC, bool upperO
 }
 
 int counter_words() { return kCounterWords; }
+int host_words_slot() { return kCounterHostWords; }
 
 // "" for the library proper; a measurement build names what it leaves out (its results are wrong by construction)
 #define FASTED_STR2(x) #x
@@ -1042,11 +1072,6 @@ hipError_t launch_padding_check(const void* points, long long ld, int n, int d, 
 
 hipError_t launch_reset_counters(unsigned long long* counters, bool keepFound, hipStream_t stream) {
     reset_counters_kernel<<<1, 256, 0, stream>>>(counters, keepFound ? 1 : 0);
-    return hipGetLastError();
-}
-
-hipError_t launch_publish_count(const unsigned long long* counters, unsigned long long* hostWords, hipStream_t stream) {
-    publish_count_kernel<<<1, 1, 0, stream>>>(counters, hostWords);
     return hipGetLastError();
 }
 

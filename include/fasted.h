@@ -73,10 +73,11 @@ void releaseResources(void);
 /* The two kernel times are HIP-event times on the stream, as the reference measures them
  * (source/findPairs.cuh:625-639,695-697); for joins of at most 512 tiles of 256 x 256, where three event records
  * would cost a third of the call, they are differences of the device's constant-rate clock, read by the kernels
- * themselves as they start (hipDeviceAttributeWallClockRate ticks). */
+ * themselves (hipDeviceAttributeWallClockRate ticks): by the first norm kernel and the join kernel as they start,
+ * and by the join kernel's last workgroup when it has nothing left to do. */
 typedef struct FastedJoinStats {
     float sumSquaredMs; /* squared-norm pre-pass (which also clears the counters): its start to the join kernel's start */
-    float joinMs;       /* the join kernel: its start to the start of what follows it on the stream */
+    float joinMs;       /* the join kernel: its start to the event behind it (small joins: to its last workgroup's report) */
     float sortMs;       /* host wall time of the row-major sort, stream synchronisation included (0 when not sorted) */
     int paddedN;        /* rows covered by the tile grid */
     int paddedD;        /* K extent the kernel looped over */
@@ -128,7 +129,11 @@ int fasted_self_join_blocked(const uint16_t* points, long long n, int d, double 
  *              workspace is used)
  *   d_pairs    room for `cap` pairs
  *   stream     hipStream_t (NULL = default stream)
- * The call synchronises the stream before returning and fills *stats.  With FASTED_SORT_PAIRS the sort's
+ * The call waits for the join before returning and fills *stats: it synchronises the stream, except that a join
+ * of at most 512 tiles of 256 x 256 returns as soon as the join kernel's last workgroup has reported the pair
+ * count to the host (a few microseconds before the stream itself reports idle, a fifth of such a call).  Every
+ * pair record and squared norm is in device memory by then, for any stream, copy or kernel that reads them next;
+ * the stream may still answer hipStreamQuery with hipErrorNotReady for a moment.  With FASTED_SORT_PAIRS the sort's
  * device buffers (a second key buffer and the radix sort's storage, about twice the bytes of the stored
  * pairs) are allocated by the library and kept for the next sort; so are the counters and, without d_sums,
  * the squared norms.  releaseResources() frees all of it.  Replaces the
