@@ -301,7 +301,8 @@ def test_pair_distances_match_fp64(fasted):
 
 def test_caller_stream_and_repeatability(fasted):
     """The device entry on a stream of the caller's: work queued on that stream before the call is seen,
-    the call returns with the stream drained, and repeated calls give the same sorted list."""
+    the call returns with the stream drained (it sorts, and the sort waits for the stream), and repeated calls
+    give the same sorted list."""
     import torch
 
     n, d = 3000, 128
@@ -318,7 +319,7 @@ def test_caller_stream_and_repeatability(fasted):
         runs = []
         for _ in range(3):
             st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, stream=stream.cuda_stream)
-            assert stream.query()  # nothing left on the stream: the call synchronised it
+            assert stream.query()  # nothing left on the stream: the sort synchronised it
             runs.append(pairs[: st.pairsStored].cpu().numpy().copy())
     torch.cuda.synchronize()
     assert st.pairsFound == st_want.pairsFound
@@ -508,3 +509,38 @@ def test_small_joins_time_themselves_with_the_device_clock(fasted):
              for _ in range(10))
     per_tile_small, per_tile_big = best / 1.0, tb / 3.0  # one round of the 256 workgroups against three
     assert 1.0 / 3.0 < per_tile_small / per_tile_big < 3.0, (best, tb)
+
+
+def test_small_join_results_are_complete_for_a_reader_on_another_stream(fasted):
+    """A join of at most 512 tiles returns when the join kernel's last workgroup has reported to the host, before
+    the stream reports idle.  The pair records and the squared norms must be in device memory by then for a reader
+    that is not ordered behind the join's stream: each of many unsorted joins on the default stream is read back
+    at once through a copy on a second, non-blocking stream, from a buffer that was overwritten in between."""
+    import torch
+
+    n, d = 4096, 128
+    bits = datasets.uniform_bytes(n, d, seed=321)
+    eps = datasets.epsilon_for_neighbours(bits, 24)
+    want, st_want, sums_want = device_join(fasted, bits, eps)  # sorted, fully synchronised
+    pts = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    cap = int(st_want.pairsFound) + 1024
+    pairs = torch.empty((cap, 2), dtype=torch.int32, device="cuda")
+    sums = torch.empty(n, dtype=torch.float32, device="cuda")
+    host_pairs = torch.empty((cap, 2), dtype=torch.int32).pin_memory()
+    host_sums = torch.empty(n, dtype=torch.float32).pin_memory()
+    reader = torch.cuda.Stream()  # default priority
+    key = lambda a: a[:, 0].astype(np.int64) * n + a[:, 1]
+    want_keys = key(want)
+    for it in range(100):
+        pairs.fill_(-1)
+        sums.fill_(-1.0)
+        torch.cuda.synchronize()
+        st = fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, sums_ptr=sums.data_ptr(), flags=0)
+        with torch.cuda.stream(reader):
+            host_pairs.copy_(pairs, non_blocking=True)
+            host_sums.copy_(sums, non_blocking=True)
+        reader.synchronize()
+        assert st.pairsFound == st_want.pairsFound == st.pairsStored, it
+        got = host_pairs[: st.pairsStored].numpy()
+        assert np.array_equal(np.sort(key(got)), want_keys), it
+        assert np.array_equal(host_sums.numpy(), sums_want), it
