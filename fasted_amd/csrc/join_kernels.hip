@@ -345,11 +345,12 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
         __syncthreads();
         if (threadIdx.x != 0) return;
         if (atomicAdd(&p.counters[kCounterDone], 1ull) + 1 != gridDim.x) return;
+        const unsigned long long through = wall_clock64() | 1ull;  // every workgroup is through (never 0)
         __hip_atomic_store(&hostWords[0], atomicAdd(&p.counters[kCounterFound], 0ull), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_SYSTEM);
         __hip_atomic_store(&hostWords[1], p.counters[kCounterStampNorms], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // both are on their way before the word that the host watches
-        __hip_atomic_store(&hostWords[3], wall_clock64() | 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(&hostWords[3], through, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     };
 
     // set by the kernel that formed this join's per-point halves: some point has a non-finite squared norm
