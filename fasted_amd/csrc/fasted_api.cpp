@@ -84,7 +84,8 @@ struct Workspace {
 
     void ensure(size_t n) {
         if (!hostCount) {
-            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocDefault));
+            // coherent whatever the environment says: the host watches these words while the kernel still runs
+            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&hostCount), 64, hipHostMallocCoherent));
             HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&hostCountDev), hostCount, 0));
         }
         if (!counters) {
@@ -263,7 +264,7 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     // last workgroup when it hands the pair count to the host.  Larger joins, and the entry
     // that owns no pinned memory, are timed with events on the stream as the reference is
     // (source/findPairs.cuh:625-639,695-697,728-736).
-    const bool stamped = !fixed && fasted::tile_count(q.n, c.n) <= 512;
+    const bool stamped = !fixed && !(flags & FASTED_EVENT_TIMING) && fasted::tile_count(q.n, c.n) <= 512;
     const bool events = !stamped && stats != nullptr;
     if (events) HIP_CHECK(hipEventRecord(t.ev[0], stream));
     if (!(flags & FASTED_SKIP_SUMS)) {

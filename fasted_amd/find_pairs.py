@@ -14,6 +14,7 @@ FASTED_SORT_PAIRS = 1
 FASTED_NO_EPILOGUE = 2
 FASTED_SKIP_SUMS = 4
 FASTED_SYMMETRIC = 8
+FASTED_EVENT_TIMING = 16
 
 
 def compute_selectivity(result_set_size: int, dataset_size: int) -> float:

@@ -92,11 +92,15 @@ enum {
     FASTED_SORT_PAIRS = 1,  /* sort stored pairs row-major, as source/pair.cuh:151-158 */
     FASTED_NO_EPILOGUE = 2, /* measurement only: run the contraction, skip test + emit */
     FASTED_SKIP_SUMS = 4,   /* d_sums already holds the squared norms */
-    FASTED_SYMMETRIC = 8    /* self-join only, off by default: dist(q,c) = dist(c,q), so compute only the tiles
+    FASTED_SYMMETRIC = 8,   /* self-join only, off by default: dist(q,c) = dist(c,q), so compute only the tiles
                                on and above the diagonal and emit both orientations of every pair found there.
                                Same pair set, about half the matrix-core work; the reference always computes the
                                full matrix (source/findPairs.cuh:650-653), which is also this library's default
                                and what its TFLOPS figure assumes. */
+    FASTED_EVENT_TIMING = 16 /* time the kernels with HIP events and wait for the stream whatever the size of the
+                               join, as the reference does (source/findPairs.cuh:625-639,695-697): for joins of at
+                               most 512 tiles this costs the call about 15 us and is what a profiler's kernel
+                               durations compare with. */
 };
 
 /* Host buffers in, host buffers out.  `points` is N x D row-major IEEE binary16 bit

@@ -501,6 +501,15 @@ def test_small_joins_time_themselves_with_the_device_clock(fasted):
         assert st.sumSquaredMs + st.joinMs < wall_ms
         best = st.joinMs if best is None else min(best, st.joinMs)
     assert 0.003 < best < 0.2, best  # 256 tiles of two slabs: some tens of microseconds
+    # the same join timed with events on the stream (FASTED_EVENT_TIMING): the dispatch as the command processor
+    # sees it, a little longer than first instruction to last sign-off, and the same pairs
+    from fasted_amd import find_pairs as fp
+
+    timed = [fasted.self_join_device(pts.data_ptr(), n, d, d, eps, pairs.data_ptr(), cap, flags=fp.FASTED_EVENT_TIMING)
+             for _ in range(10)]
+    assert all(t.pairsFound == st.pairsFound for t in timed)
+    by_events = min(t.joinMs for t in timed)
+    assert 0.5 * best < by_events < 5.0 * best, (best, by_events)
     # event-timed neighbour: 6000 points = 576 tiles
     big = datasets.exponential(6000, d, seed=3)
     ptsb = torch.from_numpy(big.view(np.int16).copy()).cuda()
