@@ -324,8 +324,9 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     const int2* const sStage = reinterpret_cast<const int2*>(lds + kLdsStage) + wave * kWaveStagePairs;  // this wave's region
 
     // (timing of small joins: the first workgroup notes when the kernel started, straight into the host's words)
+    auto host_words = [&]() { return reinterpret_cast<unsigned long long*>(p.counters[kCounterHostWords]); };
     if (blockIdx.x == 0 && threadIdx.x == 0) {
-        unsigned long long* const hostWords = reinterpret_cast<unsigned long long*>(p.counters[kCounterHostWords]);
+        unsigned long long* const hostWords = host_words();
         if (hostWords) __hip_atomic_store(&hostWords[2], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 
@@ -339,11 +340,13 @@ __global__ void __launch_bounds__(kThreads, 1) join_kernel(JoinParams p) {
     // pair counter are over by then as well -- their old values have come back and been used -- so the last to
     // sign off reads the final count.
     auto sign_off = [&]() {
-        unsigned long long* const hostWords = reinterpret_cast<unsigned long long*>(p.counters[kCounterHostWords]);
+        unsigned long long* const hostWords = host_words();
         if (!hostWords) return;
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
         __syncthreads();
-        if (threadIdx.x != 0) return;
+        // (Not `threadIdx.x != 0`: the thread number would stay in a vector register until here, across the tile
+        // loop, and move the accumulators and the MFMA operand tuples off their 4-register alignment.)
+        if (wave != 0 || lane_now() != 0) return;
         if (atomicAdd(&p.counters[kCounterDone], 1ull) + 1 != gridDim.x) return;
         const unsigned long long through = wall_clock64() | 1ull;  // every workgroup is through (never 0)
         __hip_atomic_store(&hostWords[0], atomicAdd(&p.counters[kCounterFound], 0ull), __ATOMIC_RELAXED,
