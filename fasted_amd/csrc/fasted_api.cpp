@@ -319,7 +319,13 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
             std::atomic_thread_fence(std::memory_order_acquire);
         }
         if (!reported) HIP_CHECK(hipStreamSynchronize(stream));
-        cnt[0] = w[0];
+        if (w[3] != 0) {
+            cnt[0] = w[0];
+        } else {
+            // the stream has drained without a report (a counter block that names no host words): the count is
+            // still where the kernel keeps it
+            HIP_CHECK(hipMemcpy(cnt, counters, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+        }
     }
     cnt[1] = (jl.epilogue && cnt[0] > cap) ? cap : cnt[0];
     cnt[2] = fasted::tile_count(q.n, c.n);
@@ -341,8 +347,9 @@ void join_on_device(PointSet q, PointSet c, bool selfJoin, int d, double epsilon
     if (stats) {
         if (stamped) {
             const volatile unsigned long long* const w = g_ws.hostCount;  // [1] norms start, [2] join start, [3] join over
-            stats->sumSquaredMs = (float)((double)(w[2] - w[1]) / g_ws.clockKHz());
-            stats->joinMs = (float)((double)(w[3] - w[2]) / g_ws.clockKHz());
+            const bool reportedTimes = w[3] != 0;  // (no report, no clock readings: the times stay 0)
+            stats->sumSquaredMs = reportedTimes ? (float)((double)(w[2] - w[1]) / g_ws.clockKHz()) : 0.f;
+            stats->joinMs = reportedTimes ? (float)((double)(w[3] - w[2]) / g_ws.clockKHz()) : 0.f;
         } else {
             stats->sumSquaredMs = t.ms(0, 1);
             stats->joinMs = t.ms(1, 2);
